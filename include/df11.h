@@ -1,0 +1,137 @@
+/*
+ * df11.h -- C-ABI of the MI355X (gfx950) DFloat11 weight-decompression path.
+ *
+ * Two shared libraries export these symbols:
+ *   libdf11_hip.so    device entry points (section "Device"), needs the HIP runtime
+ *   libdf11_codec.so  host-only codec (section "Host codec"), plain C++
+ *
+ * Conventions: every function returns DF11_OK (0) or a negative DF11_ERR_*
+ * code; df11_error_string() names it.  The library never allocates or frees
+ * device memory and never synchronises the device: kernels are enqueued on the
+ * caller's stream and the caller owns every buffer until that work completes.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ */
+#ifndef DF11_H
+#define DF11_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DF11_OK 0
+#define DF11_ERR_INVALID_ARGUMENT (-1)
+#define DF11_ERR_UNSUPPORTED (-2)
+#define DF11_ERR_HIP (-3)           /* a HIP runtime call failed; see df11_last_hip_error() */
+#define DF11_ERR_CAPACITY (-4)      /* an output buffer is too small */
+#define DF11_ERR_FORMAT (-5)        /* the code cannot be expressed in the DF11 LUT layout */
+
+/* Format constants (reference: dfloat11/dfloat11.py:45-46). */
+#define DF11_BYTES_PER_THREAD 8
+#define DF11_THREADS_PER_BLOCK 512
+#define DF11_BLOCK_BYTES 4096
+#define DF11_GAP_BYTES_PER_BLOCK 320
+#define DF11_MAX_ELEMS_PER_BLOCK 32768
+
+int df11_version(void);
+const char *df11_error_string(int code);
+
+/* ------------------------------------------------------------------ Device */
+
+/* Text of the last HIP error seen by this library on the calling thread. */
+const char *df11_last_hip_error(void);
+
+/*
+ * Size in bytes of the derived decode tables for one compressed tensor.
+ * The tables depend only on `luts`; build them once per tensor (at load time)
+ * and keep them next to it.  No counterpart in the reference, whose kernel
+ * chases the byte LUTs in global memory on every symbol (decode.cu:105-116).
+ */
+size_t df11_tables_bytes(void);
+
+/*
+ * Derive the multi-symbol decode tables from the DF11 byte LUTs.
+ *   luts    device, u8[n_luts][256]: rows 0..n_luts-2 hierarchical decode LUTs,
+ *           row n_luts-1 code lengths (layout: dfloat11_utils.py:68-115)
+ *   tables  device, df11_tables_bytes() bytes, 16-byte aligned
+ */
+int df11_build_tables(const uint8_t *luts, int32_t n_luts, void *tables, void *stream);
+
+/*
+ * Decode one DF11 stream into BF16.  Replaces the reference's kernel launch
+ *   _decode(grid, block, shared_mem, args=[luts, encoded_exponent, sign_mantissa,
+ *           output_positions, gaps, reconstructed, n_luts, n_bytes, n_elements])
+ * (dfloat11/dfloat11.py:139-151; kernel signature dfloat11/decode.cu:25-34).
+ * The six pointers and three sizes keep the reference's order and meaning;
+ * sizes are 64-bit here.  All pointers are device pointers.
+ *   output_positions  u32[ceil(n_bytes/4096)] at least (the entry after the
+ *                     last block is not read)
+ *   gaps              u8[320 * ceil(n_bytes/4096)]
+ *   max_elems_per_block  max(diff(output_positions)), what the reference keeps
+ *                     as (shared_mem_size - 2052) / 2 (dfloat11.py:301-306);
+ *                     <= 0 selects the format's worst case (32768)
+ *   tables            from df11_build_tables() for the same luts
+ */
+int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint8_t *sign_mantissa,
+                const uint32_t *output_positions, const uint8_t *gaps, uint16_t *outputs,
+                int32_t n_luts, int64_t n_bytes, int64_t n_elements,
+                int32_t max_elems_per_block, const void *tables, void *stream);
+
+/* -------------------------------------------------------------- Host codec */
+
+/*
+ * Exponent histogram of n BF16 words: hist[e] = #{ i : (w[i] >> 7) & 0xFF == e }.
+ * Replaces the histogram half of get_codec (dfloat11_utils.py:24-30).
+ */
+int df11_histogram(const uint16_t *w, int64_t n, uint64_t hist[256], int32_t n_threads);
+
+/*
+ * Prefix code for the exponent bytes: optimal (Huffman) including one
+ * end-of-stream leaf of weight 1, limited to 32 bits, and shaped so that the
+ * DF11 LUT layout can express it (at most 16 sub-tables; symbols >= 240 only
+ * on the fourth LUT level).  code_len[s] == 0 for absent symbols.
+ * Replaces HuffmanCodec.from_frequencies + get_32bit_codec
+ * (dfloat11_utils.py:32, 37-65).
+ */
+int df11_build_code(const uint64_t hist[256], uint8_t code_len[256], uint32_t code_val[256],
+                    int32_t *eof_len, uint32_t *eof_val);
+
+/*
+ * Hierarchical byte LUTs + length row for a code (get_luts,
+ * dfloat11_utils.py:68-115).  luts has room for cap_rows rows of 256 bytes;
+ * *n_luts receives the row count (decode rows + 1).
+ */
+int df11_build_luts(const uint8_t code_len[256], const uint32_t code_val[256],
+                    uint8_t *luts, int32_t cap_rows, int32_t *n_luts);
+
+/* Split BF16 words into exponent bytes and sign|mantissa bytes (dfloat11_utils.py:175-178). */
+int df11_split(const uint16_t *w, int64_t n, uint8_t *exponent, uint8_t *sign_mantissa,
+               int32_t n_threads);
+
+/*
+ * Sizes of the encoded stream for `n` exponent bytes under a code:
+ * n_bytes (encoded_exponent), n_blocks = ceil(n_bytes/4096).
+ */
+int df11_encode_size(const uint8_t *exponent, int64_t n, const uint8_t code_len[256],
+                     int64_t *n_bytes, int64_t *n_blocks, int32_t n_threads);
+
+/*
+ * Bit-pack the exponent bytes MSB-first and emit the per-thread gaps and
+ * per-block output positions (encode, dfloat11_utils.py:118-170).
+ *   encoded           u8[n_bytes]            from df11_encode_size
+ *   gaps              u8[320 * n_blocks]
+ *   output_positions  u32[n_blocks + 1]      always n_blocks + 1 entries
+ * The final partial byte is padded with the leading bits of the end-of-stream
+ * code, as the reference does.
+ */
+int df11_encode(const uint8_t *exponent, int64_t n, const uint8_t code_len[256],
+                const uint32_t code_val[256], int32_t eof_len, uint32_t eof_val,
+                uint8_t *encoded, int64_t n_bytes, uint8_t *gaps, uint32_t *output_positions,
+                int64_t n_blocks, int32_t n_threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DF11_H */

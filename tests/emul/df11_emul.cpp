@@ -1,0 +1,148 @@
+// Host emulation of the decode kernel's data flow, for bounds-checked testing
+// without a GPU.  It calls the very functions the gfx950 kernel calls
+// (dfloat11_amd/csrc/df11_core.h) in the same order -- table build, chunk
+// fetch, count, exclusive prefix, staged emit, grouped stream-out -- one
+// "thread" after another.  Every buffer is a heap copy of exactly the size the
+// kernel is entitled to touch, so an AddressSanitizer build turns any
+// out-of-range access in the shared logic into a test failure.
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "../../dfloat11_amd/csrc/df11_core.h"
+
+using namespace df11;
+
+namespace {
+// Heap block of exactly n elements: malloc gives a 16-byte aligned start and,
+// under AddressSanitizer, a red zone that begins right after the last byte.
+template <class T>
+struct Exact {
+  T* p;
+  explicit Exact(size_t n) : p(static_cast<T*>(malloc(n * sizeof(T) ? n * sizeof(T) : 1))) {}
+  ~Exact() { free(p); }
+  Exact(const Exact&) = delete;
+};
+}  // namespace
+
+extern "C" int df11_emul_tables(const uint8_t* luts, int n_luts, uint8_t* tables) {
+  const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
+  std::vector<uint8_t> rows((size_t)(n_rows + 1) * 256);
+  memcpy(rows.data(), luts, (size_t)n_rows * 256);
+  memcpy(rows.data() + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
+  Luts l{rows.data(), n_rows};
+  for (uint32_t idx = 0; idx < (uint32_t)kTableEntries; ++idx) {
+    uint32_t e = make_dec_entry(l, idx);
+    memcpy(tables + kDecOffset + 4 * idx, &e, 4);
+    tables[kCntFullOffset + idx] = make_cnt_full_entry(l, idx);
+    tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
+  }
+  return 0;
+}
+
+// Same arguments as df11_decode (include/df11.h), host pointers; `grid` plays
+// gridDim.x.  n_positions/n_gap_bytes/out_elems size the bounds-checked copies.
+extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
+                                const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
+                                int n_luts, int64_t n_bytes, int64_t n_elements,
+                                int max_elems_per_block, int grid, int codes_misalign,
+                                int out_misalign) {
+  if (max_elems_per_block <= 0 || max_elems_per_block > kMaxElemsPerBlock)
+    max_elems_per_block = kMaxElemsPerBlock;
+  const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  const int stage_cap = ((max_elems_per_block + 8 + 15) / 16) * 16;
+  const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
+
+  // exact-size copies of everything the kernel may read
+  Exact<uint8_t> c_codes((size_t)n_bytes + codes_misalign);
+  uint8_t* codes_p = c_codes.p + codes_misalign;
+  memcpy(codes_p, codes, (size_t)n_bytes);
+  Exact<uint8_t> c_sm((size_t)n_elements + out_misalign);
+  uint8_t* sm_p = c_sm.p + out_misalign;
+  memcpy(sm_p, sign_mantissa, (size_t)n_elements);
+  Exact<uint32_t> c_pos((size_t)n_blocks);
+  memcpy(c_pos.p, positions, (size_t)n_blocks * 4);
+  Exact<uint8_t> c_gaps((size_t)n_blocks * kGapBytesPerBlock);
+  memcpy(c_gaps.p, gaps, (size_t)n_blocks * kGapBytesPerBlock);
+  Exact<uint16_t> c_out((size_t)n_elements + out_misalign);
+  uint16_t* out_p = c_out.p + out_misalign;
+  memset(c_out.p, 0xEE, ((size_t)n_elements + out_misalign) * 2);
+  Exact<uint8_t> tables((size_t)kTablesBytes);
+  df11_emul_tables(luts, n_luts, tables.p);
+  Exact<uint8_t> rows((size_t)(n_rows + 1) * 256);
+  memcpy(rows.p, luts, (size_t)n_rows * 256);
+  memcpy(rows.p + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
+  Exact<uint8_t> stage((size_t)stage_cap);
+
+  const Tables t{reinterpret_cast<const uint32_t*>(tables.p + kDecOffset), tables.p + kCntFullOffset,
+                 tables.p + kCntTailOffset};
+  const Luts l{rows.p, n_rows};
+  const bool codes_aligned = (reinterpret_cast<uintptr_t>(codes_p) & 7) == 0;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(sm_p) & 7) == 0 &&
+                      (reinterpret_cast<uintptr_t>(out_p) & 15) == 0;
+  const int64_t n_gap_bytes = n_blocks * kGapBytesPerBlock;
+
+  std::vector<Chunk> chunk(kThreads);
+  std::vector<uint32_t> gap(kThreads), count(kThreads);
+  for (int wg = 0; wg < grid; ++wg) {
+    for (int64_t blk = wg; blk < n_blocks; blk += grid) {
+      uint32_t total = 0;
+      for (int tid = 0; tid < kThreads; ++tid) {
+        const int64_t gid = blk * kThreads + tid;
+        chunk[tid] = fetch_chunk(codes_p, n_bytes, gid, codes_aligned);
+        gap[tid] = gap_of(c_gaps.p, gid, n_gap_bytes);
+        count[tid] = count_chunk(t, l, chunk[tid].hi, chunk[tid].lo, chunk[tid].next, gap[tid]);
+        total += count[tid];
+      }
+      const BlockPlan p = plan_block((int64_t)c_pos.p[blk], total, n_elements, stage_cap);
+      memset(stage.p, 0xDD, (size_t)stage_cap);
+      uint32_t excl = 0;
+      for (int tid = 0; tid < kThreads; ++tid) {
+        const uint32_t quota = thread_quota(excl, count[tid], p.n_out);
+        // a thread with nothing to write may hold an out-of-range pointer; it must not use it
+        emit_chunk(t, l, chunk[tid].hi, chunk[tid].lo, chunk[tid].next, gap[tid], quota,
+                   quota ? stage.p + p.phase + excl : nullptr);
+        excl += count[tid];
+      }
+      const uint32_t n_groups = n_groups_of(p);
+      for (uint32_t g = 0; g < n_groups; ++g) stream_group(g, p, stage.p, sm_p, out_p, vec_ok);
+    }
+  }
+  memcpy(out, out_p, (size_t)n_elements * 2);
+  return 0;
+}
+
+#ifdef DF11_EMUL_MAIN
+// Stand-alone driver (built with AddressSanitizer): reads one case from a file
+//   i64 n_luts, n_bytes, n_elements, n_blocks, max_elems, grid, codes_misalign, out_misalign
+//   luts | codes | sign_mantissa | positions (n_blocks u32) | gaps
+// and writes the decoded u16 words to the output file.
+#include <cstdio>
+int main(int argc, char** argv) {
+  if (argc != 3) return 2;
+  FILE* f = fopen(argv[1], "rb");
+  if (!f) return 2;
+  int64_t h[8];
+  if (fread(h, 8, 8, f) != 8) return 2;
+  const int64_t n_luts = h[0], n_bytes = h[1], n_elements = h[2], n_blocks = h[3];
+  Exact<uint8_t> luts((size_t)n_luts * 256), codes((size_t)n_bytes), sm((size_t)n_elements);
+  Exact<uint32_t> pos((size_t)n_blocks);
+  Exact<uint8_t> gaps((size_t)n_blocks * kGapBytesPerBlock);
+  Exact<uint16_t> out((size_t)n_elements);
+  bool ok = fread(luts.p, 1, (size_t)n_luts * 256, f) == (size_t)n_luts * 256 &&
+            fread(codes.p, 1, (size_t)n_bytes, f) == (size_t)n_bytes &&
+            fread(sm.p, 1, (size_t)n_elements, f) == (size_t)n_elements &&
+            fread(pos.p, 4, (size_t)n_blocks, f) == (size_t)n_blocks &&
+            fread(gaps.p, 1, (size_t)n_blocks * kGapBytesPerBlock, f) == (size_t)n_blocks * kGapBytesPerBlock;
+  fclose(f);
+  if (!ok) return 2;
+  int rc = df11_emul_decode(luts.p, codes.p, sm.p, pos.p, gaps.p, out.p, (int)n_luts, n_bytes,
+                            n_elements, (int)h[4], (int)h[5], (int)h[6], (int)h[7]);
+  if (rc) return 3;
+  FILE* g = fopen(argv[2], "wb");
+  if (!g) return 2;
+  fwrite(out.p, 2, (size_t)n_elements, g);
+  fclose(g);
+  return 0;
+}
+#endif

@@ -1,0 +1,141 @@
+"""Runs the decode kernel's shared host/device logic (dfloat11_amd/csrc/df11_core.h)
+on the CPU, thread by thread, against the oracle -- with exact-size buffers and,
+for a subset, under AddressSanitizer.  This is where indexing mistakes are meant
+to surface before anything is launched on a GPU."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from tests.df11_cases import KINDS, compress_product, make_case, max_elems_per_block
+
+EMUL_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
+
+
+@pytest.fixture(scope="module")
+def emul():
+    subprocess.run(["make", "-s", "-C", EMUL_DIR], check=True)
+    L = ctypes.CDLL(os.path.join(EMUL_DIR, "libdf11_emul.so"))
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.df11_emul_decode.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, i32, i32]
+    L.df11_emul_decode.restype = i32
+    return L
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0):
+    n = c["sign_mantissa"].size
+    out = np.zeros(n, np.uint16)
+    luts = np.ascontiguousarray(c["luts"])
+    rc = L.df11_emul_decode(_p(luts), _p(c["encoded_exponent"]), _p(c["sign_mantissa"]),
+                            _p(c["output_positions"]), _p(c["gaps"]), _p(out), luts.shape[0],
+                            c["encoded_exponent"].size, n, max_elems, grid, codes_misalign, out_misalign)
+    assert rc == 0
+    return out
+
+
+def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=None):
+    n = c["sign_mantissa"].size
+    n_bytes = c["encoded_exponent"].size
+    n_blocks = -(-n_bytes // 4096)
+    luts = np.ascontiguousarray(c["luts"])
+    inp, outp = str(tmp_path / "case.bin"), str(tmp_path / "out.bin")
+    with open(inp, "wb") as f:
+        f.write(np.array([luts.shape[0], n_bytes, n, n_blocks, max_elems, grid, codes_misalign,
+                          out_misalign], np.int64).tobytes())
+        f.write(luts.tobytes())
+        f.write(c["encoded_exponent"].tobytes())
+        f.write(c["sign_mantissa"].tobytes())
+        f.write(np.ascontiguousarray(c["output_positions"][:n_blocks]).tobytes())
+        f.write(c["gaps"].tobytes())
+    res = subprocess.run([os.path.join(EMUL_DIR, "df11_emul_asan"), inp, outp],
+                         capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-3000:]
+    return np.fromfile(outp, dtype=np.uint16)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("n", [1, 2, 511, 4097, 60_000])
+def test_emulated_kernel_matches_oracle(emul, oracle, kind, n):
+    w = make_case(kind, n, 31)
+    c = compress_product(w)
+    ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                          c["output_positions"], c["gaps"])
+    assert np.array_equal(ref, w)
+    got = run_emul(emul, c, max_elems=max_elems_per_block(c["output_positions"]))
+    assert np.array_equal(got, ref)
+    # worst-case staging selected by max_elems <= 0
+    assert np.array_equal(run_emul(emul, c, max_elems=0, grid=1), ref)
+
+
+@pytest.mark.parametrize("kind", ["normal", "zeros", "fib", "uniform256"])
+def test_emulated_kernel_multi_block(emul, oracle, kind):
+    w = make_case(kind, 700_000, 37)
+    c = compress_product(w)
+    assert c["encoded_exponent"].size > 3 * 4096
+    got = run_emul(emul, c, max_elems=max_elems_per_block(c["output_positions"]), grid=5)
+    assert np.array_equal(got, w)
+
+
+@pytest.mark.parametrize("codes_misalign,out_misalign", [(1, 0), (0, 1), (3, 5), (4, 4)])
+def test_emulated_kernel_unaligned_pointers(emul, codes_misalign, out_misalign):
+    w = make_case("normal", 50_000, 41)
+    c = compress_product(w)
+    got = run_emul(emul, c, max_elems=max_elems_per_block(c["output_positions"]),
+                   codes_misalign=codes_misalign, out_misalign=out_misalign)
+    assert np.array_equal(got, w)
+
+
+def test_emulated_kernel_reads_reference_streams(emul, oracle):
+    """Streams written by the oracle's restatement of the reference encoder
+    (dahuffman-ordered table, reference LUT fill, positions possibly one short)."""
+    w = make_case("outliers", 90_000, 43)
+    c = oracle.compress(w)
+    n_blocks = -(-c["encoded_exponent"].size // 4096)
+    pos = np.full(n_blocks + 1, w.size, np.uint32)
+    pos[: c["output_positions"].size] = c["output_positions"]
+    c2 = dict(c, output_positions=pos)
+    assert np.array_equal(run_emul(emul, c2, max_elems=max_elems_per_block(pos)), w)
+
+
+def test_emulated_kernel_short_positions_quirk(emul, oracle):
+    from oracle.df11_oracle import EOF
+    table = {1: (8, 0b10000000), 2: (16, 0b0000000000000001), EOF: (16, 0)}
+    data = np.array([1] * 4095 + [2], np.uint8)
+    enc, gaps, pos = oracle.c_encode(data, table)
+    luts = np.zeros((3, 256), np.uint8)
+    luts[0, :] = 1
+    luts[0, 0] = 255
+    luts[1, :] = 2
+    luts[2, 1], luts[2, 2] = 8, 16
+    sm = (np.arange(data.size) % 251).astype(np.uint8)
+    # the kernel reads one position per block: entry 1 is the reference's sentinel
+    c = dict(luts=luts, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps)
+    assert pos.size == 2 and -(-enc.size // 4096) == 2
+    assert np.array_equal(run_emul(emul, c), oracle.merge_bf16(data, sm))
+
+
+def test_emulated_kernel_small_staging_is_clamped_not_overrun(emul, tmp_path):
+    """A caller that understates max_elems_per_block loses elements but never
+    writes outside the staging area (checked under AddressSanitizer)."""
+    w = make_case("zeros", 100_000, 47)
+    c = compress_product(w)
+    got = run_asan(c, max_elems=1000, tmp_path=tmp_path)
+    assert got.size == w.size          # ran to completion without a sanitizer report
+
+
+@pytest.mark.parametrize("kind,n,cm,om", [("normal", 40_000, 0, 0), ("zeros", 70_000, 0, 0),
+                                          ("fib", 330_000, 0, 0), ("uniform256", 9_000, 2, 3),
+                                          ("high", 5_000, 0, 1), ("single", 1, 0, 0),
+                                          ("laplace", 4096 * 3, 7, 0)])
+def test_emulated_kernel_under_asan(emul, tmp_path, kind, n, cm, om):
+    w = make_case(kind, n, 53)
+    c = compress_product(w)
+    got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
+                   out_misalign=om, tmp_path=tmp_path)
+    assert np.array_equal(got, w)
