@@ -1,0 +1,188 @@
+"""Decode-throughput benchmark of the DF11 hot path on one MI355X.
+
+A step is one decode of a Llama-3-8B-shaped decoder block (q, k, v, o, gate, up,
+down; 218 103 808 BF16 elements, random-init N(0, 0.02)) compressed as ONE DF11
+stream, from HBM-resident compressed inputs into one contiguous BF16 buffer.
+Prints one JSON line: GB/s of algorithmic traffic (compressed bytes read + BF16
+bytes written), the HBM-roofline fraction of the decode kernel, and the CPU
+oracle timed on the host cores of the same machine.
+"""
+import argparse
+import json
+import os
+import sys
+import threading
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+LLAMA3_8B_BLOCK = [("q_proj", 4096, 4096), ("k_proj", 1024, 4096), ("v_proj", 1024, 4096),
+                   ("o_proj", 4096, 4096), ("gate_proj", 14336, 4096), ("up_proj", 14336, 4096),
+                   ("down_proj", 4096, 14336)]
+
+
+def algorithmic_bytes(n_bytes, n_elements, n_luts):
+    n_blocks = -(-n_bytes // 4096)
+    return n_bytes + n_elements + 320 * n_blocks + 4 * (n_blocks + 1) + 256 * n_luts + 2 * n_elements
+
+
+def make_block(torch, device):
+    parts = []
+    for i, (_, rows, cols) in enumerate(LLAMA3_8B_BLOCK):
+        g = torch.Generator(device=device).manual_seed(1000 + i)
+        parts.append((torch.randn(rows * cols, generator=g, device=device) * 0.02).to(torch.bfloat16))
+    return torch.cat(parts)
+
+
+def cpu_baseline(stream, budget_s=12.0):
+    """Times the CPU oracle (scalar C restatement of the reference kernel) on a bounded
+    run of consecutive bitstream blocks of the same stream, on the host's cores."""
+    from oracle import df11_oracle as O
+    n_bytes = stream["encoded_exponent"].size
+    n_blocks = -(-n_bytes // 4096)
+    n_threads = max(1, min(16, len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    out = np.zeros(stream["sign_mantissa"].size, np.uint16)
+    args = (stream["luts"], stream["encoded_exponent"], stream["sign_mantissa"],
+            stream["output_positions"], stream["gaps"])
+
+    def run(b0, b1):
+        O.c_decode(*args, block_range=(b0, b1), out=out)
+
+    probe = min(n_blocks, 200)
+    t0 = time.perf_counter()
+    run(0, probe)
+    per_block_1t = (time.perf_counter() - t0) / probe
+    # whole stream if it fits the budget of CPU work, else a prefix of it; repeated so
+    # that about `budget_s` core-seconds are spent, and the median pass is reported
+    sample = int(min(n_blocks, max(n_threads, budget_s / per_block_1t)))
+    repeats = int(max(1, min(7, budget_s / (sample * per_block_1t))))
+    bounds = [sample * i // n_threads for i in range(n_threads + 1)]
+    times = []
+    for _ in range(repeats):
+        threads = [threading.Thread(target=run, args=(bounds[i], bounds[i + 1])) for i in range(n_threads)]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        times.append(time.perf_counter() - t0)
+    dt = float(np.median(times))
+    pos = stream["output_positions"].astype(np.int64)
+    elems = int(pos[min(sample, pos.size - 1)] - pos[0])
+    bytes_done = sample * (4096 + 320 + 4) + 3 * elems
+    single = bytes_done / (sample * per_block_1t)
+    return {
+        "value": bytes_done / dt / 1e9, "unit": "GB/s", "cores": n_threads, "kind": "port",
+        "sample": f"first {sample} of {n_blocks} bitstream blocks of the same stream ({elems} elements), "
+                  f"median of {repeats} passes of {dt:.2f} s, scalar C restatement of the reference "
+                  f"kernel, one thread per core over disjoint block ranges",
+        "single_thread_GBps": single / 1e9,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU only: every box has one MI355X and the decode path "
+                 "needs no exchange between GPUs; run with --gpus 1")
+
+    import torch
+    from dfloat11_amd import decode as D
+    from dfloat11_amd import dfloat11_utils as U
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w = make_block(torch, dev)
+    n_elements = w.numel()
+    w_cpu = w.cpu()
+    t0 = time.perf_counter()
+    codec, _ = U.get_codec(w_cpu)
+    luts = U.get_luts(codec.get_code_table())
+    enc, sm, pos, gaps, _ = U.encode_weights([w_cpu], codec)
+    t_encode = time.perf_counter() - t0
+    pos_np = pos.numpy().astype(np.int64)
+    max_elems = int((pos_np[1:] - pos_np[:-1]).max())
+
+    d_luts, d_enc, d_sm, d_gaps = (t.to(dev) for t in (luts, enc, sm, gaps))
+    d_pos = pos.view(torch.uint8).to(dev)
+    tables = D.build_tables(d_luts)
+    out = torch.empty(n_elements, dtype=torch.bfloat16, device=dev)
+
+    def step():
+        D.decode(d_luts, d_enc, d_sm, d_pos, d_gaps, out, tables, max_elems)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    # HIP events on the stream the kernel is launched on (torch's current stream)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        starts[i].record()
+        step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    span_ms = starts[0].elapsed_time(ends[-1])
+    ms_per_step = span_ms / a.steps
+    avg_kernel_ms = float(np.mean(kernel_ms))
+
+    bit_exact = None
+    if not a.no_verify:
+        bit_exact = bool(torch.equal(out.view(torch.int16), w.view(torch.int16)))
+
+    n_bytes = enc.numel()
+    algo = algorithmic_bytes(n_bytes, n_elements, luts.shape[0])
+    value = algo / (ms_per_step * 1e-3) / 1e9
+    achieved = algo / (avg_kernel_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "decode GB/s (bytes in+out)", "value": value, "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {
+            "workload": "Llama-3-8B-shaped decoder block (q,k,v,o,gate,up,down) as one DF11 stream, "
+                        "random-init N(0,0.02) BF16, decoded into one contiguous buffer",
+            "n_elements": n_elements, "encoded_exponent_bytes": n_bytes,
+            "bitstream_blocks": -(-n_bytes // 4096), "n_luts": int(luts.shape[0]),
+            "algorithmic_bytes_per_step": algo, "bytes_per_element": algo / n_elements,
+            "compressed_over_bf16": (n_bytes + n_elements + gaps.numel() + 4 * pos.numel()) / (2 * n_elements),
+            "max_elems_per_block": max_elems, "bit_exact": bit_exact,
+            "encode_seconds_host": t_encode, "wall_ms_per_step": wall * 1e3 / a.steps,
+            "kernel_ms_min": float(np.min(kernel_ms)), "kernel_ms_max": float(np.max(kernel_ms)),
+        },
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "decode_kernel", "avg_launch_ms": avg_kernel_ms},
+    }
+    if not a.no_cpu_baseline:
+        stream = dict(luts=luts.numpy(), encoded_exponent=enc.numpy(), sign_mantissa=sm.numpy(),
+                      output_positions=pos.numpy(), gaps=gaps.numpy())
+        result["cpu_baseline"] = cpu_baseline(stream)
+    if bit_exact is False:
+        result["error"] = "decoded block differs from the original"
+    print(json.dumps(result))
+    if bit_exact is False:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

@@ -9,6 +9,7 @@
 // carries its own LUTs.
 #include <algorithm>
 #include <array>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <queue>
@@ -37,6 +38,18 @@ struct Leaf {
 int pick_threads(int32_t requested, int64_t n, int64_t min_per_thread) {
   int hw = (int)std::thread::hardware_concurrency();
   if (hw <= 0) hw = 1;
+  // hardware_concurrency() reports the machine, not the share this process may
+  // use; honour the usual environment knobs and stay modest by default.
+  for (const char* name : {"DF11_NUM_THREADS", "OMP_NUM_THREADS"}) {
+    if (const char* v = std::getenv(name)) {
+      const int k = std::atoi(v);
+      if (k > 0) {
+        hw = k;
+        break;
+      }
+    }
+  }
+  if (hw > 64) hw = 64;
   int t = requested > 0 ? requested : hw;
   int64_t cap = n / min_per_thread;
   if (cap < 1) cap = 1;

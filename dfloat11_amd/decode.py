@@ -1,0 +1,65 @@
+"""Thin torch-facing wrappers over the device C-ABI (include/df11.h).
+
+torch is used for device memory and streams only; the work happens in
+libdf11_hip.so.  There is no CPU path: these functions raise if the tensors are
+not on a GPU or the library cannot be loaded.
+"""
+import torch
+
+from . import _native
+
+
+def _stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(**tensors):
+    for name, t in tensors.items():
+        if not t.is_cuda:
+            raise _native.DF11Error(f"{name} must live on the GPU (got {t.device}); there is no CPU decode path")
+        if not t.is_contiguous():
+            raise _native.DF11Error(f"{name} must be contiguous")
+
+
+def tables_bytes():
+    return int(_native.hip_lib().df11_tables_bytes())
+
+
+def build_tables(luts, out=None):
+    """Derive the multi-symbol decode tables for `luts` (u8 [n_luts, 256], on the GPU)."""
+    _require_cuda(luts=luts)
+    if luts.dtype != torch.uint8 or luts.dim() != 2 or luts.shape[1] != 256 or luts.shape[0] < 2:
+        raise _native.DF11Error(f"luts must be uint8 [n_luts >= 2, 256], got {luts.dtype} {tuple(luts.shape)}")
+    if out is None:
+        out = torch.empty(tables_bytes(), dtype=torch.uint8, device=luts.device)
+    with torch.cuda.device(luts.device):
+        rc = _native.hip_lib().df11_build_tables(luts.data_ptr(), luts.shape[0], out.data_ptr(),
+                                                 _stream_ptr(luts.device))
+    _native.check(rc, "df11_build_tables")
+    return out
+
+
+def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, tables,
+           max_elems_per_block=0):
+    """Decode one DF11 stream into `out` (bfloat16, >= n_elements) on the current stream."""
+    _require_cuda(luts=luts, encoded_exponent=encoded_exponent, sign_mantissa=sign_mantissa,
+                  output_positions=output_positions, gaps=gaps, out=out, tables=tables)
+    n_elements = sign_mantissa.numel()
+    n_bytes = encoded_exponent.numel()
+    n_blocks = -(-n_bytes // 4096)
+    if out.dtype != torch.bfloat16 or out.numel() < n_elements:
+        raise _native.DF11Error("out must be a bfloat16 tensor with at least n_elements elements")
+    if output_positions.numel() * output_positions.element_size() < 4 * n_blocks:
+        raise _native.DF11Error("output_positions shorter than one entry per bitstream block")
+    if gaps.numel() < 320 * n_blocks:
+        raise _native.DF11Error("gaps shorter than 320 bytes per bitstream block")
+    if tables.numel() * tables.element_size() < tables_bytes():
+        raise _native.DF11Error("tables buffer too small")
+    with torch.cuda.device(out.device):
+        rc = _native.hip_lib().df11_decode(
+            luts.data_ptr(), encoded_exponent.data_ptr(), sign_mantissa.data_ptr(),
+            output_positions.data_ptr(), gaps.data_ptr(), out.data_ptr(),
+            luts.shape[0], n_bytes, n_elements, int(max_elems_per_block), tables.data_ptr(),
+            _stream_ptr(out.device))
+    _native.check(rc, "df11_decode")
+    return out

@@ -1,0 +1,57 @@
+"""The C-ABI libraries load and export every symbol include/df11.h declares (no GPU calls)."""
+import ctypes
+import os
+import re
+
+from dfloat11_amd import _native, build
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "df11.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(df11_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    names = _declared()
+    assert "df11_decode" in names and "df11_encode" in names and len(names) >= 12
+    hip = _native.hip_lib()
+    codec = _native.codec_lib()
+    for name in names:
+        assert hasattr(hip, name) or hasattr(codec, name), name
+
+
+def test_version_and_error_strings():
+    hip = _native.hip_lib()
+    assert hip.df11_version() == 1
+    assert hip.df11_error_string(0) == b"ok"
+    assert hip.df11_error_string(-1) == b"invalid argument"
+    assert hip.df11_tables_bytes() == 4096 * 4 + 4096 + 4096
+
+
+def test_argument_validation_needs_no_gpu():
+    hip = _native.hip_lib()
+    # null pointers / bad sizes are rejected before any HIP call
+    assert hip.df11_build_tables(None, 4, None, None) == -1
+    assert hip.df11_decode(None, None, None, None, None, None, 4, 100, 100, 0, None, None) == -1
+    assert hip.df11_decode(None, None, None, None, None, None, 4, -1, 100, 0, None, None) == -1
+    # empty streams decode to nothing
+    assert hip.df11_decode(None, None, None, None, None, None, 4, 0, 0, 0, None, None) == 0
+
+
+def test_decode_without_gpu_fails_loudly():
+    import pytest
+    import torch
+    from dfloat11_amd import decode
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    t = torch.zeros(2, 256, dtype=torch.uint8)
+    with pytest.raises(_native.DF11Error):
+        decode.build_tables(t)
+
+
+def test_libraries_are_in_tree():
+    assert os.path.dirname(build.HIP_LIB) == os.path.join(ROOT, "dfloat11_amd")
+    assert os.path.exists(build.HIP_LIB) and os.path.exists(build.CODEC_LIB)

@@ -1,0 +1,183 @@
+"""Parity of the HIP decode path (through the C-ABI) with the CPU oracle, on a real MI355X."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from dfloat11_amd import decode as D
+from tests.df11_cases import KINDS, compress_product, make_case, max_elems_per_block
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def to_gpu(c, pad_front=0):
+    """Upload the five stream tensors.  pad_front > 0 shifts every buffer by that many
+    bytes from its allocation start to exercise the unaligned paths."""
+    def up(a):
+        a = np.ascontiguousarray(a)
+        t = torch.empty(a.nbytes + pad_front, dtype=torch.uint8, device=DEV)
+        t[pad_front:].copy_(torch.from_numpy(a.view(np.uint8).reshape(-1)))
+        return t[pad_front:]
+    g = {k: up(c[k]) for k in ("luts", "encoded_exponent", "sign_mantissa", "gaps")}
+    g["luts"] = g["luts"].view(-1, 256)
+    g["output_positions"] = torch.from_numpy(np.ascontiguousarray(c["output_positions"]).view(np.uint8)).to(DEV)
+    return g
+
+
+def gpu_decode(c, max_elems=None, pad_front=0, out=None):
+    g = to_gpu(c, pad_front)
+    n = c["sign_mantissa"].size
+    tables = D.build_tables(g["luts"].contiguous())
+    if out is None:
+        out = torch.full((n,), float("nan"), dtype=torch.bfloat16, device=DEV)
+    if max_elems is None:
+        max_elems = max_elems_per_block(c["output_positions"])
+    D.decode(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
+             out, tables, max_elems)
+    torch.cuda.synchronize()
+    return out.view(torch.int16).cpu().numpy().view(np.uint16)[:n]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("n", [1, 2, 511, 4097, 300_000])
+def test_gpu_matches_oracle(oracle, kind, n):
+    print(f"case kind={kind} n={n}", flush=True)
+    w = make_case(kind, n, 61)
+    c = compress_product(w)
+    ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                          c["output_positions"], c["gaps"])
+    got = gpu_decode(c)
+    assert np.array_equal(got, ref)
+    assert np.array_equal(got, w)
+
+
+@pytest.mark.parametrize("kind", ["normal", "zeros", "fib"])
+def test_gpu_worst_case_staging(kind):
+    print(f"case worst-case staging kind={kind}", flush=True)
+    w = make_case(kind, 200_000, 67)
+    c = compress_product(w)
+    assert np.array_equal(gpu_decode(c, max_elems=0), w)
+
+
+def test_gpu_tables_match_host_build():
+    print("case tables", flush=True)
+    emul_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
+    lib_path = os.path.join(emul_dir, "libdf11_emul.so")
+    if not os.path.exists(lib_path):
+        subprocess.run(["make", "-s", "-C", emul_dir, "libdf11_emul.so"], check=True)
+    L = ctypes.CDLL(lib_path)
+    for kind in ("normal", "fib", "uniform256", "high"):
+        c = compress_product(make_case(kind, 400_000, 71))
+        luts = np.ascontiguousarray(c["luts"])
+        host = np.zeros(D.tables_bytes(), np.uint8)
+        L.df11_emul_tables(luts.ctypes.data_as(ctypes.c_void_p), luts.shape[0],
+                           host.ctypes.data_as(ctypes.c_void_p))
+        dev = D.build_tables(torch.from_numpy(luts).to(DEV))
+        torch.cuda.synchronize()
+        assert np.array_equal(dev.cpu().numpy(), host), kind
+
+
+@pytest.mark.parametrize("pad", [1, 2, 4, 7])
+def test_gpu_unaligned_inputs(pad):
+    print(f"case unaligned pad={pad}", flush=True)
+    w = make_case("normal", 120_000, 73)
+    c = compress_product(w)
+    assert np.array_equal(gpu_decode(c, pad_front=pad), w)
+
+
+def test_gpu_unaligned_output():
+    print("case unaligned output", flush=True)
+    w = make_case("laplace", 120_000, 79)
+    c = compress_product(w)
+    buf = torch.zeros(w.size + 16, dtype=torch.bfloat16, device=DEV)
+    for shift in (1, 3, 8):
+        buf.zero_()
+        got = gpu_decode(c, out=buf[shift:shift + w.size])
+        assert np.array_equal(got, w)
+        whole = buf.view(torch.int16).cpu().numpy()
+        assert not whole[:shift].any() and not whole[shift + w.size:].any()
+
+
+def test_gpu_reads_reference_encoder_streams(oracle):
+    """Streams laid out by the oracle's restatement of the reference encoder."""
+    print("case reference-encoder stream", flush=True)
+    w = make_case("outliers", 250_000, 83)
+    c = oracle.compress(w)
+    n_blocks = -(-c["encoded_exponent"].size // 4096)
+    pos = np.full(n_blocks + 1, w.size, np.uint32)
+    pos[: c["output_positions"].size] = c["output_positions"]
+    c = dict(c, output_positions=pos)
+    assert np.array_equal(gpu_decode(c), w)
+
+
+def test_gpu_does_not_write_outside_output():
+    print("case guard bands", flush=True)
+    w = make_case("normal", 77_777, 89)
+    c = compress_product(w)
+    guard = 4096
+    buf = torch.full((w.size + 2 * guard,), 1.0, dtype=torch.bfloat16, device=DEV)
+    got = gpu_decode(c, out=buf[guard:guard + w.size])
+    assert np.array_equal(got, w)
+    whole = buf.view(torch.int16).cpu().numpy()
+    assert (whole[:guard] == 0x3F80).all() and (whole[guard + w.size:] == 0x3F80).all()
+
+
+def test_gpu_side_stream_and_repeat():
+    print("case side stream", flush=True)
+    w1 = make_case("normal", 500_000, 97)
+    w2 = make_case("laplace", 300_000, 101)
+    c1, c2 = compress_product(w1), compress_product(w2)
+    g1, g2 = to_gpu(c1), to_gpu(c2)
+    t1, t2 = D.build_tables(g1["luts"]), D.build_tables(g2["luts"])
+    out = torch.empty(max(w1.size, w2.size), dtype=torch.bfloat16, device=DEV)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        for _ in range(3):   # same output buffer reused, stream order is the only guard
+            D.decode(g1["luts"], g1["encoded_exponent"], g1["sign_mantissa"], g1["output_positions"],
+                     g1["gaps"], out, t1, max_elems_per_block(c1["output_positions"]))
+            a = out[: w1.size].clone()
+            D.decode(g2["luts"], g2["encoded_exponent"], g2["sign_mantissa"], g2["output_positions"],
+                     g2["gaps"], out, t2, max_elems_per_block(c2["output_positions"]))
+            b = out[: w2.size].clone()
+    s.synchronize()
+    assert np.array_equal(a.view(torch.int16).cpu().numpy().view(np.uint16), w1)
+    assert np.array_equal(b.view(torch.int16).cpu().numpy().view(np.uint16), w2)
+
+
+def test_gpu_full_size_linear_round_trip():
+    """4096x4096 N(0, 0.02): encode -> decode is the identity (size-independent property)."""
+    print("case 4096x4096", flush=True)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    w = (torch.randn(4096, 4096, generator=g) * 0.02).to(torch.bfloat16)
+    wu = w.view(torch.int16).numpy().view(np.uint16).reshape(-1)
+    c = compress_product(wu)
+    assert c["sign_mantissa"].size == 16_777_216
+    got = gpu_decode(c)
+    assert np.array_equal(got, wu)
+
+
+def test_gpu_llama_block_round_trip():
+    """Llama-3-8B-shaped decoder block compressed as one stream: 218 103 808 elements."""
+    print("case llama block", flush=True)
+    shapes = [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096), (4096, 14336)]
+    parts = []
+    for i, (r, cdim) in enumerate(shapes):
+        g = torch.Generator(device=DEV).manual_seed(1000 + i)
+        parts.append((torch.randn(r * cdim, generator=g, device=DEV) * 0.02).to(torch.bfloat16))
+    w = torch.cat(parts)
+    assert w.numel() == 218_103_808
+    wu = w.view(torch.int16).cpu().numpy().view(np.uint16)
+    c = compress_product(wu)
+    g = to_gpu(c)
+    tables = D.build_tables(g["luts"])
+    out = torch.empty_like(w)
+    D.decode(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
+             out, tables, max_elems_per_block(c["output_positions"]))
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), w.view(torch.int16))
