@@ -92,6 +92,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a 256 MiB streaming copy kernel 5 times (profiler byte-counter calibration)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU only: every box has one MI355X and the decode path "
@@ -128,6 +130,13 @@ def main():
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
+    if a.calibration_copy:
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            D.calibration_copy(src, dst)
+        torch.cuda.synchronize()
+        del src, dst
     # HIP events on the stream the kernel is launched on (torch's current stream)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps)]

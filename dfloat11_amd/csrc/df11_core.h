@@ -19,19 +19,20 @@ constexpr int kBlockBytes = kChunkBytes * kThreads;
 constexpr int kGapBytesPerBlock = kThreads * 5 / 8;
 constexpr int kMaxElemsPerBlock = kBlockBytes * 8;   // one-bit codes
 
-// Width of the direct-indexed tables: one lookup resolves every code that
-// ends inside the next kK bits of the stream.
-constexpr int kK = 12;
+// Width of the direct-indexed table: one lookup resolves up to four codes that
+// end inside the next kK bits of the stream.
+constexpr int kK = 11;
 constexpr int kTableEntries = 1 << kK;
 
 // Derived table blob (built once per tensor from the byte LUTs):
-//   dec  u32[4096]  up to three symbols that end inside the 12-bit window:
-//                   sym0 | sym1<<8 | sym2<<16 | bits<<24 | count<<28 ; 0 = first code longer than 12 bits
-//   cntf u8[4096]   all codes that end inside the window: count<<4 | bits ; 0 = as above
-//   cntt u8[4096]   index (1<<r)|v, v = the next r bits (r < 12): how many codes start inside those r bits
+//   dec  u32[2048][2]  word 0: the symbols of up to four codes that end inside the
+//                      11-bit window, first code in byte 0;
+//                      word 1 ("meta"): bits consumed in byte 0, code count in
+//                      byte 1; 0 = the first code is longer than 11 bits
+//   cntt u8[2048]      index (1<<r)|v, v = the next r bits (r < 11): how many codes
+//                      start inside those r bits
 constexpr int kDecOffset = 0;
-constexpr int kCntFullOffset = kTableEntries * 4;
-constexpr int kCntTailOffset = kCntFullOffset + kTableEntries;
+constexpr int kCntTailOffset = kTableEntries * 8;
 constexpr int kTablesBytes = kCntTailOffset + kTableEntries;
 
 // Byte LUT rows a pointer entry can name: values 255..240 name rows 1..16.
@@ -61,32 +62,37 @@ DF11_HD void walk(const Luts& l, uint64_t window, uint32_t& sym, uint32_t& len) 
 
 // ---- table construction (one entry per call) --------------------------------
 
-DF11_HD uint32_t make_dec_entry(const Luts& l, uint32_t idx) {
+// Is the code at the top of `window` settled by its first `known` bits alone?
+// The byte LUTs answer for any 8-bit index, including indices whose low bits
+// are not known yet; the answer counts only if it uses no more than the known
+// bits AND does not change when the unknown bits do.  The second condition
+// rejects slots that merely inherited a neighbour's symbol (the end-of-stream
+// code's slots, unused code space): there the symbol found with the unknown
+// bits at 0 and at 1 differs, or its length exceeds the known bits.
+DF11_HD bool resolve(const Luts& l, uint64_t window, uint32_t known, uint32_t& sym, uint32_t& len) {
+  if (known == 0) return false;
+  const uint64_t unknown_mask = known >= 64u ? 0ull : (~0ull >> known);
+  uint32_t s0, n0, s1, n1;
+  walk(l, window & ~unknown_mask, s0, n0);
+  walk(l, window | unknown_mask, s1, n1);
+  sym = s0;
+  len = n0;
+  return n0 <= known && s0 == s1 && n0 == n1;
+}
+
+DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_t& meta) {
   const uint64_t window = (uint64_t)idx << (64 - kK);
-  uint32_t pos = 0, k = 0, syms = 0;
-  while (k < 3) {
+  uint32_t pos = 0, k = 0;
+  syms = 0;
+  while (k < 4) {
     uint32_t s, n;
-    walk(l, window << pos, s, n);
-    if (pos + n > (uint32_t)kK) break;
+    if (!resolve(l, window << pos, (uint32_t)kK - pos, s, n)) break;
     syms |= s << (8 * k);
     pos += n;
     ++k;
   }
-  return k ? (syms | (pos << 24) | (k << 28)) : 0u;
-}
-
-DF11_HD uint8_t make_cnt_full_entry(const Luts& l, uint32_t idx) {
-  const uint64_t window = (uint64_t)idx << (64 - kK);
-  uint32_t pos = 0, k = 0;
-  for (;;) {
-    uint32_t s, n;
-    walk(l, window << pos, s, n);
-    if (pos + n > (uint32_t)kK) break;
-    pos += n;
-    ++k;
-    if (pos == (uint32_t)kK) break;
-  }
-  return (uint8_t)((k << 4) | pos);   // k <= 12, pos <= 12
+  meta = k ? (pos | (k << 8)) : 0u;
+  if (!k) syms = 0;
 }
 
 DF11_HD uint8_t make_cnt_tail_entry(const Luts& l, uint32_t idx) {
@@ -98,96 +104,142 @@ DF11_HD uint8_t make_cnt_tail_entry(const Luts& l, uint32_t idx) {
   uint32_t pos = 0, k = 0;
   while (pos < (uint32_t)r) {
     uint32_t s, n;
-    walk(l, window << pos, s, n);
+    ++k;                                          // a code starts at pos
+    if (!resolve(l, window << pos, (uint32_t)r - pos, s, n)) break;   // and runs past the known bits
     pos += n;
-    ++k;
   }
   return (uint8_t)k;
 }
 
 // ---- per-chunk passes ---------------------------------------------------------
 
-struct Tables {
-  const uint32_t* dec;
-  const uint8_t* cntf;
-  const uint8_t* cntt;
+struct alignas(8) U32x2 {
+  uint32_t x, y;
 };
+struct alignas(16) U32x4 {
+  uint32_t x, y, z, w;
+};
+
+// Aligned wide access to byte buffers without type punning.
+template <class T>
+DF11_HD T load_as(const void* p) {
+  T v;
+  __builtin_memcpy(&v, __builtin_assume_aligned(p, alignof(T)), sizeof(T));
+  return v;
+}
+template <class T>
+DF11_HD void store_as(void* p, const T& v) {
+  __builtin_memcpy(__builtin_assume_aligned(p, alignof(T)), &v, sizeof(T));
+}
+
+struct Tables {
+  const uint8_t* dec;     // u32[2048][2], 8-byte aligned
+  const uint8_t* cntt;    // u8[2048]
+};
+
+// Unaligned 32-/16-bit stores (LDS supports them on gfx950; one instruction each).
+DF11_HD void store32(uint8_t* p, uint32_t v) { __builtin_memcpy(p, &v, 4); }
+DF11_HD void store16(uint8_t* p, uint32_t v) {
+  const uint16_t h = (uint16_t)v;
+  __builtin_memcpy(p, &h, 2);
+}
+
+// Keeps a rarely taken branch a branch: without it the compiler turns the body
+// into unconditional selects that every loop iteration pays for.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define DF11_KEEP_BRANCH() asm volatile("" ::: "memory")
+#else
+#define DF11_KEEP_BRANCH() ((void)0)
+#endif
+
+// The window with the 32 look-ahead bits appended below its 64 - c valid bits.
+DF11_HD uint64_t with_next(uint64_t w, uint32_t next, uint32_t c) {
+  if (c == 0) return w;
+  return w | (c >= 32u ? (uint64_t)next << (c - 32u) : (uint64_t)next >> (32u - c));
+}
+
+// Byte offset of the table entry for the top kK bits of the window.
+DF11_HD uint32_t dec_offset(uint64_t w) { return ((uint32_t)(w >> 32) >> (32 - kK - 3)) & (uint32_t)((kTableEntries - 1) * 8); }
 
 // Number of codes that start inside the 64-bit chunk {hi,lo}; `next` holds the
 // 32 stream bits after the chunk, `gap` the bit offset of the first code start.
+// Lookups stay inside the chunk (c <= 64 - kK), so the look-ahead is only needed
+// for codes longer than the table width; the last few bits are settled by one
+// lookup in the tail table.
 DF11_HD uint32_t count_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo,
                              uint32_t next, uint32_t gap) {
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
-  uint32_t c = gap, n = 0;
-  while (c < 32u) {
-    const uint32_t e = t.cntf[(uint32_t)(w >> (64 - kK))];
-    uint32_t nb;
-    if (e) {
-      n += e >> 4;
-      nb = e & 15u;
-    } else {
-      uint32_t s;
-      walk(l, w, s, nb);
-      n += 1;
+  uint32_t cn = gap;                    // byte 0: bits consumed; bits 8 and up: codes counted
+  while ((cn & 0xffu) <= 64u - (uint32_t)kK) {
+    uint32_t meta = load_as<uint32_t>(t.dec + dec_offset(w) + 4u);
+    if (meta == 0u) {
+      uint32_t s, n;
+      walk(l, with_next(w, next, cn & 0xffu), s, n);
+      meta = n | 0x100u;
+      DF11_KEEP_BRANCH();
     }
-    w <<= nb;
-    c += nb;
+    w <<= (meta & 63u);
+    cn += meta;
   }
-  w |= (uint64_t)next << (c - 32u);
-  while (c < 64u) {
-    const uint32_t r = 64u - c;
-    if (r < (uint32_t)kK) {
-      n += t.cntt[(1u << r) | (uint32_t)(w >> (64u - r))];
-      break;
-    }
-    const uint32_t e = t.cntf[(uint32_t)(w >> (64 - kK))];
-    uint32_t nb;
-    if (e) {
-      n += e >> 4;
-      nb = e & 15u;
-    } else {
-      uint32_t s;
-      walk(l, w, s, nb);
-      n += 1;
-    }
-    w <<= nb;
-    c += nb;
-  }
+  const uint32_t c = cn & 0xffu;
+  uint32_t n = cn >> 8;
+  if (c < 64u) n += t.cntt[(1u << (64u - c)) | (uint32_t)(w >> c)];
   return n;
 }
 
 // Decode the first `remaining` codes of the chunk and write their symbols
-// (exponent bytes) to stage[0..remaining).
+// (exponent bytes) to p[0..remaining).  While four or more bytes remain the
+// four symbol bytes of a lookup are stored at once: bytes past the codes it
+// resolved are overwritten by the next store.  The last one to three symbols
+// are gathered in a register and stored exactly, so nothing is ever written at
+// or beyond p + remaining.
 DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo, uint32_t next,
-                        uint32_t gap, uint32_t remaining, uint8_t* stage) {
+                        uint32_t gap, uint32_t remaining, uint8_t* p) {
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
-  uint32_t c = gap;
-  bool refilled = false;
-  while (remaining) {
-    if (!refilled && c >= 32u) {
+  uint32_t c = gap;                     // bit 7 is set once the look-ahead has been appended
+  uint32_t rem = remaining;
+  while (rem >= 4u) {
+    if (c - 32u < 96u) {                // 32 <= c < 128: room for the look-ahead, not yet appended
       w |= (uint64_t)next << (c - 32u);
-      refilled = true;
+      c += 128u;
+      DF11_KEEP_BRANCH();
     }
-    const uint32_t e = t.dec[(uint32_t)(w >> (64 - kK))];
-    uint32_t nb;
-    if (e) {
-      const uint32_t k = e >> 28;
-      nb = (e >> 24) & 15u;
-      stage[0] = (uint8_t)e;
-      if (k > 1u && remaining > 1u) stage[1] = (uint8_t)(e >> 8);
-      if (k > 2u && remaining > 2u) stage[2] = (uint8_t)(e >> 16);
-      const uint32_t take = k < remaining ? k : remaining;
-      stage += take;
-      remaining -= take;
-    } else {
-      uint32_t s;
-      walk(l, w, s, nb);
-      stage[0] = (uint8_t)s;
-      stage += 1;
-      remaining -= 1;
+    const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+    uint32_t syms = e.x, meta = e.y;
+    if (meta == 0u) {
+      uint32_t n;
+      walk(l, w, syms, n);              // at least 32 valid bits: c < 32, or already appended
+      meta = n | 0x100u;
+      DF11_KEEP_BRANCH();
     }
-    w <<= nb;
-    c += nb;
+    store32(p, syms);
+    const uint32_t k = meta >> 8;
+    p += k;
+    rem -= k;
+    w <<= (meta & 63u);
+    c += meta & 0xffu;
+  }
+  if (rem) {
+    uint32_t acc = 0, got = 0;          // got: bits gathered, 8 per symbol
+    while (got < 8u * rem) {
+      if (c - 32u < 96u) {
+        w |= (uint64_t)next << (c - 32u);
+        c += 128u;
+      }
+      const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+      uint32_t syms = e.x, meta = e.y;
+      if (meta == 0u) {
+        uint32_t n;
+        walk(l, w, syms, n);
+        meta = n | 0x100u;
+      }
+      acc |= syms << got;
+      got += 8u * (meta >> 8);
+      w <<= (meta & 63u);
+      c += meta & 0xffu;
+    }
+    if (rem & 2u) store16(p, acc);
+    if (rem & 1u) p[rem & 2u] = (uint8_t)(acc >> (8u * (rem & 2u)));
   }
 }
 
@@ -212,25 +264,6 @@ struct Chunk {
   uint32_t hi, lo, next;
 };
 
-struct alignas(8) U32x2 {
-  uint32_t x, y;
-};
-struct alignas(16) U32x4 {
-  uint32_t x, y, z, w;
-};
-
-// Aligned wide access to byte buffers without type punning.
-template <class T>
-DF11_HD T load_as(const void* p) {
-  T v;
-  __builtin_memcpy(&v, __builtin_assume_aligned(p, alignof(T)), sizeof(T));
-  return v;
-}
-template <class T>
-DF11_HD void store_as(void* p, const T& v) {
-  __builtin_memcpy(__builtin_assume_aligned(p, alignof(T)), &v, sizeof(T));
-}
-
 DF11_HD Chunk fetch_chunk(const uint8_t* codes, int64_t n_bytes, int64_t gid, bool aligned) {
   const int64_t off = gid * kChunkBytes;
   uint32_t d0 = 0, d1 = 0, d2 = 0;
@@ -250,17 +283,20 @@ DF11_HD Chunk fetch_chunk(const uint8_t* codes, int64_t n_bytes, int64_t gid, bo
 }
 
 // Where a bitstream block lands.  The staging area keeps the output's phase
-// modulo 8 elements (staging index i holds output element a0 + i), so that
-// 8-byte staging reads pair with 8-byte sign|mantissa loads and 16-byte stores.
+// modulo 16 elements (staging index i holds output element a0 + i), so that
+// 16-byte staging reads pair with 16-byte sign|mantissa loads and 32 bytes of
+// BF16 stores.
 struct BlockPlan {
-  int64_t a0;       // output index of staging index 0 (multiple of 8)
-  uint32_t phase;   // staging index of the block's first element, 0..7
+  int64_t a0;       // output index of staging index 0 (multiple of 16)
+  uint32_t phase;   // staging index of the block's first element, 0..15
   uint32_t n_out;   // elements this block produces (clamped to n_elements and to the staging capacity)
 };
 
+constexpr int kGroup = 16;   // elements per lane per write-out step
+
 DF11_HD BlockPlan plan_block(int64_t base, uint32_t total, int64_t n_elements, int32_t stage_cap) {
   BlockPlan p;
-  p.a0 = base & ~(int64_t)7;
+  p.a0 = base & ~(int64_t)(kGroup - 1);
   p.phase = (uint32_t)(base - p.a0);
   int64_t end = base + (int64_t)total;
   if (end > n_elements) end = n_elements;
@@ -278,35 +314,53 @@ DF11_HD uint32_t thread_quota(uint32_t excl, uint32_t count, uint32_t n_out) {
   return my_end > excl ? my_end - excl : 0u;
 }
 
-DF11_HD uint32_t n_groups_of(const BlockPlan& p) { return (p.phase + p.n_out + 7u) >> 3; }
-
-// bytes 0,1 (or 2,3) of x moved to the low bytes of the two 16-bit halves
-DF11_HD uint32_t spread_lo(uint32_t x) { return (x & 0xffu) | ((x & 0xff00u) << 8); }
-DF11_HD uint32_t spread_hi(uint32_t x) { return ((x >> 16) & 0xffu) | ((x >> 8) & 0xff0000u); }
-DF11_HD uint32_t merge2(uint32_t e, uint32_t m) {   // two BF16 words per 32-bit word
-  return ((m & 0x00800080u) << 8) | (e << 7) | (m & 0x007f007fu);
+DF11_HD uint32_t n_groups_of(const BlockPlan& p) {
+  return (p.phase + p.n_out + (uint32_t)kGroup - 1u) / (uint32_t)kGroup;
 }
 
-// Write output group g of the block: elements a0 + 8g .. a0 + 8g + 7 that
-// belong to the block.  `vec_ok`: sign_mantissa is 8-byte and out 16-byte aligned.
-DF11_HD void stream_group(uint32_t g, const BlockPlan& p, const uint8_t* stage,
-                          const uint8_t* sign_mantissa, uint16_t* out, bool vec_ok) {
+// Four BF16 words from four exponent bytes E and four sign|mantissa bytes S:
+// high bytes (S & 0x80) | (E >> 1), low bytes (E << 7) | (S & 0x7f), interleaved.
+DF11_HD void merge4(uint32_t E, uint32_t S, uint32_t& out01, uint32_t& out23) {
+  const uint32_t hi = (S & 0x80808080u) | ((E >> 1) & 0x7f7f7f7fu);
+  const uint32_t lo = ((E << 7) & 0x80808080u) | (S & 0x7f7f7f7fu);
+#if defined(__HIP_DEVICE_COMPILE__)
+  out01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);   // lo0 hi0 lo1 hi1
+  out23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);   // lo2 hi2 lo3 hi3
+#else
+  out01 = (lo & 0xffu) | ((hi & 0xffu) << 8) | ((lo & 0xff00u) << 8) | ((hi & 0xff00u) << 16);
+  out23 = ((lo >> 16) & 0xffu) | ((hi >> 8) & 0xff00u) | ((lo >> 8) & 0xff0000u) | (hi & 0xff000000u);
+#endif
+}
+
+// True when group g of the block can take the 16-wide path.
+DF11_HD bool group_is_full(uint32_t g, const BlockPlan& p) {
+  const uint32_t s0 = g * (uint32_t)kGroup;
+  return s0 >= p.phase && s0 + (uint32_t)kGroup <= p.phase + p.n_out;
+}
+
+// 16-wide path: `m` holds the 16 sign|mantissa bytes of the group (loaded by the
+// caller, possibly long before), staging bytes come from `stage`.
+DF11_HD void stream_group_full(uint32_t g, const BlockPlan& p, const uint8_t* stage, const U32x4& m,
+                               uint16_t* out) {
+  const uint32_t s0 = g * (uint32_t)kGroup;
+  const U32x4 e = load_as<U32x4>(stage + s0);
+  U32x4 o0, o1;
+  merge4(e.x, m.x, o0.x, o0.y);
+  merge4(e.y, m.y, o0.z, o0.w);
+  merge4(e.z, m.z, o1.x, o1.y);
+  merge4(e.w, m.w, o1.z, o1.w);
+  store_as<U32x4>(out + p.a0 + s0, o0);
+  store_as<U32x4>(out + p.a0 + s0 + 8, o1);
+}
+
+// Element-wise path for the ragged ends of a block (and for unaligned buffers).
+DF11_HD void stream_group_ragged(uint32_t g, const BlockPlan& p, const uint8_t* stage,
+                                 const uint8_t* sign_mantissa, uint16_t* out) {
   const uint32_t first = p.phase, last = p.phase + p.n_out;
-  const uint32_t s0 = g << 3;
-  if (vec_ok && s0 >= first && s0 + 8u <= last) {
-    const U32x2 e8 = load_as<U32x2>(stage + s0);
-    const U32x2 m8 = load_as<U32x2>(sign_mantissa + p.a0 + s0);
-    U32x4 o;
-    o.x = merge2(spread_lo(e8.x), spread_lo(m8.x));
-    o.y = merge2(spread_hi(e8.x), spread_hi(m8.x));
-    o.z = merge2(spread_lo(e8.y), spread_lo(m8.y));
-    o.w = merge2(spread_hi(e8.y), spread_hi(m8.y));
-    store_as<U32x4>(out + p.a0 + s0, o);
-  } else {
-    const uint32_t lo_i = s0 > first ? s0 : first;
-    const uint32_t hi_i = s0 + 8u < last ? s0 + 8u : last;
-    for (uint32_t i = lo_i; i < hi_i; ++i) out[p.a0 + i] = merge(stage[i], sign_mantissa[p.a0 + i]);
-  }
+  const uint32_t s0 = g * (uint32_t)kGroup;
+  const uint32_t lo_i = s0 > first ? s0 : first;
+  const uint32_t hi_i = s0 + (uint32_t)kGroup < last ? s0 + (uint32_t)kGroup : last;
+  for (uint32_t i = lo_i; i < hi_i; ++i) out[p.a0 + i] = merge(stage[i], sign_mantissa[p.a0 + i]);
 }
 
 }  // namespace df11

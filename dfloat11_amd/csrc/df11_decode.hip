@@ -4,16 +4,17 @@
 // bitstream block at a time and walks the grid persistently, so the derived
 // tables are copied into LDS once per workgroup rather than once per block.
 // Per block:
-//   1. every thread fetches its 8-byte chunk (+4 bytes of look-ahead) and its
-//      5-bit gap, and counts the codes starting in the chunk with the
-//      multi-symbol count tables (LDS);
+//   1. every thread takes its 8-byte chunk (+4 bytes of look-ahead) and 5-bit gap
+//      (fetched one block ahead) and counts the codes starting in the chunk with
+//      the four-symbol table in LDS;
 //   2. exclusive prefix sum of the 512 counts: DPP scan inside each wavefront,
 //      eight wavefront totals combined through LDS;
-//   3. every thread decodes its codes again with the three-symbol table and
-//      writes exponent bytes into an LDS staging area laid out in output order;
-//   4. the workgroup streams the staging area out: 8 exponent bytes (LDS) +
-//      8 sign|mantissa bytes (global, coalesced) -> one 16-byte BF16 store per
-//      lane.
+//   3. every thread decodes its codes again and stores the symbols of each lookup
+//      with one unaligned 32-bit LDS store into a staging area laid out in output
+//      order;
+//   4. the workgroup streams the staging area out: 16 exponent bytes (LDS) + 16
+//      sign|mantissa bytes (global, coalesced, requested before step 1) -> two
+//      16-byte BF16 stores per lane.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -48,8 +49,9 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const uint8_t* __rest
     rows[n_rows * 256 + i] = luts[(n_luts - 1) * 256 + i];
   __syncthreads();
   Luts l{rows, n_rows};
-  reinterpret_cast<uint32_t*>(tables + kDecOffset)[idx] = make_dec_entry(l, idx);
-  tables[kCntFullOffset + idx] = make_cnt_full_entry(l, idx);
+  uint32_t syms, meta;
+  make_dec_entry(l, idx, syms, meta);
+  reinterpret_cast<uint2*>(tables + kDecOffset)[idx] = make_uint2(syms, meta);
   tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
 }
 
@@ -90,7 +92,7 @@ struct DecodeArgs {
   int32_t n_luts;
   int32_t stage_cap;      // bytes of staging, multiple of 16
   int32_t codes_aligned;  // codes pointer is 8-byte aligned
-  int32_t vec_ok;         // sign_mantissa 8-byte aligned and out 16-byte aligned
+  int32_t vec_ok;         // sign_mantissa and out both 16-byte aligned
 };
 
 __global__ __launch_bounds__(kThreads) void decode_kernel(const DecodeArgs a) {
@@ -115,15 +117,33 @@ __global__ __launch_bounds__(kThreads) void decode_kernel(const DecodeArgs a) {
   }
   __syncthreads();
 
-  const Tables t{reinterpret_cast<const uint32_t*>(lds_tables + kDecOffset),
-                 lds_tables + kCntFullOffset, lds_tables + kCntTailOffset};
+  const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
   const Luts l{lds_rows, n_rows};
   const int64_t n_gap_bytes = a.n_blocks * kGapBytesPerBlock;
+  const bool vec_ok = a.vec_ok != 0;
 
-  for (int64_t blk = blockIdx.x; blk < a.n_blocks; blk += gridDim.x) {
-    const int64_t gid = blk * kThreads + tid;
-    const Chunk c = fetch_chunk(a.codes, a.n_bytes, gid, a.codes_aligned != 0);
-    const uint32_t gap = gap_of(a.gaps, gid, n_gap_bytes);
+  int64_t blk = blockIdx.x;
+  Chunk c = fetch_chunk(a.codes, a.n_bytes, blk * kThreads + tid, a.codes_aligned != 0);
+  uint32_t gap = gap_of(a.gaps, blk * kThreads + tid, n_gap_bytes);
+
+  for (; blk < a.n_blocks; blk += gridDim.x) {
+    // ---- requests whose latency the two decode passes hide: the next block's
+    // chunk and gap, and this block's sign|mantissa bytes for the write-out
+    const int64_t next_blk = blk + gridDim.x;
+    Chunk c_next{0, 0, 0};
+    uint32_t gap_next = 0;
+    if (next_blk < a.n_blocks) {
+      c_next = fetch_chunk(a.codes, a.n_bytes, next_blk * kThreads + tid, a.codes_aligned != 0);
+      gap_next = gap_of(a.gaps, next_blk * kThreads + tid, n_gap_bytes);
+    }
+    const int64_t base = (int64_t)a.positions[blk];
+    const int64_t a0 = base & ~(int64_t)(kGroup - 1);
+    U32x4 m0{0, 0, 0, 0}, m1{0, 0, 0, 0};
+    if (vec_ok) {
+      const int64_t i0 = a0 + (int64_t)tid * kGroup, i1 = i0 + (int64_t)kThreads * kGroup;
+      if (i0 + kGroup <= a.n_elements) m0 = load_as<U32x4>(a.sign_mantissa + i0);
+      if (i1 + kGroup <= a.n_elements) m1 = load_as<U32x4>(a.sign_mantissa + i1);
+    }
 
     // ---- pass 1: how many codes start in my chunk
     const uint32_t count = count_chunk(t, l, c.hi, c.lo, c.next, gap);
@@ -142,17 +162,38 @@ __global__ __launch_bounds__(kThreads) void decode_kernel(const DecodeArgs a) {
     const uint32_t excl = wave_base + incl - count;
 
     // ---- pass 2: decode into the staging area, in output order
-    const BlockPlan p = plan_block((int64_t)a.positions[blk], total, a.n_elements, a.stage_cap);
+    const BlockPlan p = plan_block(base, total, a.n_elements, a.stage_cap);
     emit_chunk(t, l, c.hi, c.lo, c.next, gap, thread_quota(excl, count, p.n_out),
                stage + p.phase + excl);
     __syncthreads();
 
-    // ---- stream out: 8 elements per lane per step
+    // ---- stream out, 16 elements per lane per step.  No barrier is needed after
+    // this: the next block's staging writes come after its prefix-sum barrier,
+    // which every wavefront reaches only when it is done reading here.
     const uint32_t n_groups = n_groups_of(p);
-    for (uint32_t g = tid; g < n_groups; g += kThreads)
-      stream_group(g, p, stage, a.sign_mantissa, a.out, a.vec_ok != 0);
-    __syncthreads();   // staging and wave_sums are reused by the next block
+    for (uint32_t g = tid; g < n_groups; g += kThreads) {
+      if (vec_ok && group_is_full(g, p)) {
+        U32x4 m;
+        if (g == (uint32_t)tid) m = m0;
+        else if (g == (uint32_t)(tid + kThreads)) m = m1;
+        else m = load_as<U32x4>(a.sign_mantissa + p.a0 + (int64_t)g * kGroup);
+        stream_group_full(g, p, stage, m, a.out);
+      } else {
+        stream_group_ragged(g, p, stage, a.sign_mantissa, a.out);
+      }
+    }
+    c = c_next;
+    gap = gap_next;
   }
+}
+
+// Plain streaming copy, 16 bytes per lane: the known-traffic kernel against
+// which hardware byte counters are calibrated.
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src,
+                                                   uint4* __restrict__ dst, int64_t n_vec) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
 }
 
 struct DeviceInfo {
@@ -211,6 +252,19 @@ int df11_build_tables(const uint8_t* luts, int32_t n_luts, void* tables, void* s
   return e == hipSuccess ? DF11_OK : hip_fail(e);
 }
 
+int df11_calibration_copy(const void* src, void* dst, int64_t n_bytes, void* stream) {
+  if (!src || !dst || n_bytes <= 0 || (n_bytes & 15)) return DF11_ERR_INVALID_ARGUMENT;
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15)
+    return DF11_ERR_INVALID_ARGUMENT;
+  DeviceInfo info;
+  if (int rc = device_info(info)) return rc;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)(info.cus * 8)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint4*>(src),
+                     static_cast<uint4*>(dst), n_bytes / 16);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? DF11_OK : hip_fail(e);
+}
+
 int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
                 const uint32_t* output_positions, const uint8_t* gaps, uint16_t* outputs,
                 int32_t n_luts, int64_t n_bytes, int64_t n_elements, int32_t max_elems_per_block,
@@ -240,9 +294,9 @@ int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint
   a.n_elements = n_elements;
   a.n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
   a.n_luts = n_luts;
-  a.stage_cap = ((max_elems_per_block + 8 + 15) / 16) * 16;   // + up to 7 elements of output phase
+  a.stage_cap = ((max_elems_per_block + kGroup + 15) / 16) * 16;   // + up to 15 elements of output phase
   a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
-  a.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
+  a.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 15) == 0 &&
              (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
 
   const size_t lds_bytes = (size_t)kFixedLds + (size_t)a.stage_cap;

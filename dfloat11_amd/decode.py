@@ -63,3 +63,15 @@ def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, t
             _stream_ptr(out.device))
     _native.check(rc, "df11_decode")
     return out
+
+
+def calibration_copy(src, dst):
+    """Streaming copy of known size (profiler byte-counter calibration)."""
+    _require_cuda(src=src, dst=dst)
+    n = src.numel() * src.element_size()
+    if dst.numel() * dst.element_size() != n:
+        raise _native.DF11Error("src and dst differ in size")
+    with torch.cuda.device(src.device):
+        rc = _native.hip_lib().df11_calibration_copy(src.data_ptr(), dst.data_ptr(), n, _stream_ptr(src.device))
+    _native.check(rc, "df11_calibration_copy")
+    return dst

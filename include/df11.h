@@ -79,6 +79,13 @@ int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint
                 int32_t n_luts, int64_t n_bytes, int64_t n_elements,
                 int32_t max_elems_per_block, const void *tables, void *stream);
 
+/*
+ * Streaming device copy of n_bytes (multiple of 16, both pointers 16-byte
+ * aligned).  Measurement aid with no counterpart in the reference: a kernel of
+ * known HBM traffic against which profiler byte counters are calibrated.
+ */
+int df11_calibration_copy(const void *src, void *dst, int64_t n_bytes, void *stream);
+
 /* -------------------------------------------------------------- Host codec */
 
 /*

@@ -32,9 +32,9 @@ extern "C" int df11_emul_tables(const uint8_t* luts, int n_luts, uint8_t* tables
   memcpy(rows.data() + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
   Luts l{rows.data(), n_rows};
   for (uint32_t idx = 0; idx < (uint32_t)kTableEntries; ++idx) {
-    uint32_t e = make_dec_entry(l, idx);
-    memcpy(tables + kDecOffset + 4 * idx, &e, 4);
-    tables[kCntFullOffset + idx] = make_cnt_full_entry(l, idx);
+    uint32_t e[2];
+    make_dec_entry(l, idx, e[0], e[1]);
+    memcpy(tables + kDecOffset + 8 * idx, e, 8);
     tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
   }
   return 0;
@@ -50,7 +50,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   if (max_elems_per_block <= 0 || max_elems_per_block > kMaxElemsPerBlock)
     max_elems_per_block = kMaxElemsPerBlock;
   const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
-  const int stage_cap = ((max_elems_per_block + 8 + 15) / 16) * 16;
+  const int stage_cap = ((max_elems_per_block + kGroup + 15) / 16) * 16;
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
 
   // exact-size copies of everything the kernel may read
@@ -74,11 +74,10 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   memcpy(rows.p + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
   Exact<uint8_t> stage((size_t)stage_cap);
 
-  const Tables t{reinterpret_cast<const uint32_t*>(tables.p + kDecOffset), tables.p + kCntFullOffset,
-                 tables.p + kCntTailOffset};
+  const Tables t{tables.p + kDecOffset, tables.p + kCntTailOffset};
   const Luts l{rows.p, n_rows};
   const bool codes_aligned = (reinterpret_cast<uintptr_t>(codes_p) & 7) == 0;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(sm_p) & 7) == 0 &&
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(sm_p) & 15) == 0 &&
                       (reinterpret_cast<uintptr_t>(out_p) & 15) == 0;
   const int64_t n_gap_bytes = n_blocks * kGapBytesPerBlock;
 
@@ -96,16 +95,30 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
       }
       const BlockPlan p = plan_block((int64_t)c_pos.p[blk], total, n_elements, stage_cap);
       memset(stage.p, 0xDD, (size_t)stage_cap);
-      uint32_t excl = 0;
+      // Threads of a block run concurrently on the device, so no thread may rely
+      // on a later thread repairing what it wrote.  Even blocks emit in ascending
+      // thread order, odd blocks in descending order: a store that strays into a
+      // neighbour's bytes corrupts the result in one of the two.
+      std::vector<uint32_t> excl(kThreads);
+      uint32_t run = 0;
       for (int tid = 0; tid < kThreads; ++tid) {
-        const uint32_t quota = thread_quota(excl, count[tid], p.n_out);
+        excl[tid] = run;
+        run += count[tid];
+      }
+      for (int k = 0; k < kThreads; ++k) {
+        const int tid = (blk & 1) ? kThreads - 1 - k : k;
+        const uint32_t quota = thread_quota(excl[tid], count[tid], p.n_out);
         // a thread with nothing to write may hold an out-of-range pointer; it must not use it
         emit_chunk(t, l, chunk[tid].hi, chunk[tid].lo, chunk[tid].next, gap[tid], quota,
-                   quota ? stage.p + p.phase + excl : nullptr);
-        excl += count[tid];
+                   quota ? stage.p + p.phase + excl[tid] : nullptr);
       }
       const uint32_t n_groups = n_groups_of(p);
-      for (uint32_t g = 0; g < n_groups; ++g) stream_group(g, p, stage.p, sm_p, out_p, vec_ok);
+      for (uint32_t g = 0; g < n_groups; ++g) {
+        if (vec_ok && group_is_full(g, p))
+          stream_group_full(g, p, stage.p, load_as<U32x4>(sm_p + p.a0 + (int64_t)g * kGroup), out_p);
+        else
+          stream_group_ragged(g, p, stage.p, sm_p, out_p);
+      }
     }
   }
   memcpy(out, out_p, (size_t)n_elements * 2);

@@ -28,7 +28,7 @@ def test_version_and_error_strings():
     assert hip.df11_version() == 1
     assert hip.df11_error_string(0) == b"ok"
     assert hip.df11_error_string(-1) == b"invalid argument"
-    assert hip.df11_tables_bytes() == 4096 * 4 + 4096 + 4096
+    assert hip.df11_tables_bytes() == 2048 * 8 + 2048
 
 
 def test_argument_validation_needs_no_gpu():

@@ -139,3 +139,87 @@ def test_emulated_kernel_under_asan(emul, tmp_path, kind, n, cm, om):
     got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
                    out_misalign=om, tmp_path=tmp_path)
     assert np.array_equal(got, w)
+
+
+# ---------------------------------------------------------------- derived tables
+def _host_tables(luts):
+    L = ctypes.CDLL(os.path.join(EMUL_DIR, "libdf11_emul.so"))
+    luts = np.ascontiguousarray(luts)
+    blob = np.zeros(2048 * 8 + 2048, np.uint8)
+    L.df11_emul_tables(_p(luts), luts.shape[0], _p(blob))
+    dec = blob[: 2048 * 8].view(np.uint32).reshape(2048, 2)
+    return dec, blob[2048 * 8:]
+
+
+def _first_code(bits, codes):
+    """('sym', s, len) if a code word is a prefix of `bits`; ('open',) if `bits` is
+    a proper prefix of some symbol's code word (too short to tell); ('void',) if it
+    runs into the end-of-stream code or into code space no symbol uses."""
+    for s, word in codes.items():
+        if s != "eof" and bits.startswith(word):
+            return ("sym", s, len(word))
+    if any(s != "eof" and word.startswith(bits) for s, word in codes.items()):
+        # could still become a symbol -- unless only the end-of-stream code continues it
+        return ("open",)
+    return ("void",)
+
+
+@pytest.mark.parametrize("kind,n,seed", [("normal", 300_000, 1), ("outliers", 4097, 61),
+                                         ("outliers", 200_000, 2), ("fib", 330_000, 3),
+                                         ("uniform256", 50_000, 4), ("zeros", 10_000, 5),
+                                         ("high", 3_000, 6), ("single", 100, 7)])
+def test_derived_tables_brute_force(emul, kind, n, seed):
+    """Every entry of the multi-symbol tables against the code table itself: for
+    each 11-bit pattern the first (up to four) code words that END inside it,
+    and for each shorter pattern the number of code words that START inside it.
+    Paths that run into the end-of-stream code or into unused code space are
+    exempt from there on: no valid stream contains them before its padding."""
+    c = compress_product(make_case(kind, n, seed))
+    codec = c["codec"]
+    codes = {int(s): format(int(codec.code_val[s]), "b").rjust(int(codec.code_len[s]), "0")
+             for s in range(256) if codec.code_len[s]}
+    codes["eof"] = format(codec.eof_val, "b").rjust(codec.eof_len, "0")
+    dec, cntt = _host_tables(c["luts"])
+    checked = 0
+    for idx in range(2048):
+        bits = format(idx, "011b")
+        syms, pos, void = [], 0, False
+        while len(syms) < 4:
+            r = _first_code(bits[pos:], codes)
+            if r[0] != "sym":
+                void = r[0] == "void"
+                break
+            syms.append(r[1])
+            pos += r[2]
+        word, meta = int(dec[idx, 0]), int(dec[idx, 1])
+        k, nbits = meta >> 8, meta & 0xFF
+        got = [(word >> (8 * i)) & 0xFF for i in range(k)]
+        assert got[: len(syms)] == syms, (idx, got, syms)
+        if not void:
+            checked += 1
+            assert k == len(syms) and nbits == (pos if syms else 0), (idx, meta, syms, pos)
+    assert checked > 0
+    for r in range(1, 11):
+        for v in range(1 << r):
+            bits = format(v, "b").rjust(r, "0")
+            pos, starts, void = 0, 0, False
+            while pos < r:
+                res = _first_code(bits[pos:], codes)
+                if res[0] == "void":
+                    void = True
+                    break
+                starts += 1
+                if res[0] == "open":
+                    break
+                pos += res[2]
+            if not void:
+                assert int(cntt[(1 << r) | v]) == starts, (r, bits, int(cntt[(1 << r) | v]), starts)
+
+
+@pytest.mark.parametrize("seed", range(60, 72))
+def test_emulated_kernel_long_codes_many_seeds(emul, seed):
+    """Sparse outliers give 12..14-bit codes next to 2-bit ones: the slow path and
+    the table boundaries in every position."""
+    w = make_case("outliers", 4097 + 37 * seed, seed)
+    c = compress_product(w)
+    assert np.array_equal(run_emul(emul, c, max_elems=max_elems_per_block(c["output_positions"]), grid=2), w)
