@@ -46,10 +46,11 @@ def hip_lib():
         L.df11_error_string.argtypes = [_i32]
         L.df11_error_string.restype = ctypes.c_char_p
         L.df11_last_hip_error.restype = ctypes.c_char_p
-        L.df11_tables_bytes.restype = ctypes.c_size_t
-        L.df11_build_tables.argtypes = [_vp, _i32, _vp, _vp]
-        L.df11_build_tables.restype = _i32
-        L.df11_decode.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i32, _vp, _vp]
+        L.df11_workspace_bytes.argtypes = [_i64]
+        L.df11_workspace_bytes.restype = ctypes.c_size_t
+        L.df11_prepare.argtypes = [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, ctypes.POINTER(_i32), _vp]
+        L.df11_prepare.restype = _i32
+        L.df11_decode.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp]
         L.df11_decode.restype = _i32
         L.df11_calibration_copy.argtypes = [_vp, _vp, _i64, _vp]
         L.df11_calibration_copy.restype = _i32

@@ -282,20 +282,44 @@ DF11_HD Chunk fetch_chunk(const uint8_t* codes, int64_t n_bytes, int64_t gid, bo
   return Chunk{__builtin_bswap32(d0), __builtin_bswap32(d1), __builtin_bswap32(d2)};
 }
 
-// Where a bitstream block lands.  The staging area keeps the output's phase
-// modulo 16 elements (staging index i holds output element a0 + i), so that
-// 16-byte staging reads pair with 16-byte sign|mantissa loads and 32 bytes of
+// ---- sub-blocks ------------------------------------------------------------------
+// A sub-block is the 512 bytes of bitstream that one 64-lane wavefront decodes:
+// 64 chunks, an eighth of a 4096-byte block.  The element index at which each
+// sub-block's output starts is derived once per tensor (it depends only on the
+// stream), which lets every wavefront work on its own, with no exchange between
+// the wavefronts of a workgroup.
+constexpr int kLanes = 64;
+constexpr int kSubBytes = kLanes * kChunkBytes;          // 512
+constexpr int kSubsPerBlock = kBlockBytes / kSubBytes;   // 8
+constexpr int kMaxElemsPerSub = kSubBytes * 8;           // one-bit codes
+constexpr int kGroup = 8;                                // elements per lane per write-out step
+
+// Workspace derived once per tensor: header | decode tables | sub-block positions.
+struct WorkspaceHeader {
+  uint32_t magic;
+  uint32_t n_blocks;
+  uint32_t max_sub_elems;   // largest number of elements any sub-block produces
+  uint32_t reserved[13];
+};
+constexpr uint32_t kWorkspaceMagic = 0x31314644u;   // "DF11"
+constexpr int kWsTablesOffset = 64;
+constexpr int kWsSubposOffset = kWsTablesOffset + kTablesBytes;
+DF11_HD int64_t workspace_bytes(int64_t n_blocks) {
+  return (kWsSubposOffset + 4 * (n_blocks * kSubsPerBlock + 1) + 15) & ~(int64_t)15;
+}
+
+// Where a sub-block lands.  The wavefront's staging area keeps the output's
+// phase modulo 8 elements (staging index i holds output element a0 + i), so
+// that 8-byte staging reads pair with 8-byte sign|mantissa loads and 16-byte
 // BF16 stores.
-struct BlockPlan {
-  int64_t a0;       // output index of staging index 0 (multiple of 16)
-  uint32_t phase;   // staging index of the block's first element, 0..15
-  uint32_t n_out;   // elements this block produces (clamped to n_elements and to the staging capacity)
+struct SubPlan {
+  int64_t a0;       // output index of staging index 0 (multiple of 8)
+  uint32_t phase;   // staging index of the sub-block's first element, 0..7
+  uint32_t n_out;   // elements produced (clamped to n_elements and to the staging capacity)
 };
 
-constexpr int kGroup = 16;   // elements per lane per write-out step
-
-DF11_HD BlockPlan plan_block(int64_t base, uint32_t total, int64_t n_elements, int32_t stage_cap) {
-  BlockPlan p;
+DF11_HD SubPlan plan_sub(int64_t base, uint32_t total, int64_t n_elements, int32_t stage_cap) {
+  SubPlan p;
   p.a0 = base & ~(int64_t)(kGroup - 1);
   p.phase = (uint32_t)(base - p.a0);
   int64_t end = base + (int64_t)total;
@@ -314,10 +338,6 @@ DF11_HD uint32_t thread_quota(uint32_t excl, uint32_t count, uint32_t n_out) {
   return my_end > excl ? my_end - excl : 0u;
 }
 
-DF11_HD uint32_t n_groups_of(const BlockPlan& p) {
-  return (p.phase + p.n_out + (uint32_t)kGroup - 1u) / (uint32_t)kGroup;
-}
-
 // Four BF16 words from four exponent bytes E and four sign|mantissa bytes S:
 // high bytes (S & 0x80) | (E >> 1), low bytes (E << 7) | (S & 0x7f), interleaved.
 DF11_HD void merge4(uint32_t E, uint32_t S, uint32_t& out01, uint32_t& out23) {
@@ -332,35 +352,45 @@ DF11_HD void merge4(uint32_t E, uint32_t S, uint32_t& out01, uint32_t& out23) {
 #endif
 }
 
-// True when group g of the block can take the 16-wide path.
-DF11_HD bool group_is_full(uint32_t g, const BlockPlan& p) {
-  const uint32_t s0 = g * (uint32_t)kGroup;
-  return s0 >= p.phase && s0 + (uint32_t)kGroup <= p.phase + p.n_out;
-}
+// The write-out of a sub-block splits [phase, phase + n_out) into a head of
+// fewer than 8 elements up to the first 8-aligned staging index, a body of
+// whole 8-element groups, and a tail of fewer than 8 elements.
+struct SubSpans {
+  uint32_t head_begin, head_end;   // element-wise
+  uint32_t body_begin, body_end;   // group indices (staging index / 8)
+  uint32_t tail_begin, tail_end;   // element-wise
+};
 
-// 16-wide path: `m` holds the 16 sign|mantissa bytes of the group (loaded by the
-// caller, possibly long before), staging bytes come from `stage`.
-DF11_HD void stream_group_full(uint32_t g, const BlockPlan& p, const uint8_t* stage, const U32x4& m,
-                               uint16_t* out) {
-  const uint32_t s0 = g * (uint32_t)kGroup;
-  const U32x4 e = load_as<U32x4>(stage + s0);
-  U32x4 o0, o1;
-  merge4(e.x, m.x, o0.x, o0.y);
-  merge4(e.y, m.y, o0.z, o0.w);
-  merge4(e.z, m.z, o1.x, o1.y);
-  merge4(e.w, m.w, o1.z, o1.w);
-  store_as<U32x4>(out + p.a0 + s0, o0);
-  store_as<U32x4>(out + p.a0 + s0 + 8, o1);
-}
-
-// Element-wise path for the ragged ends of a block (and for unaligned buffers).
-DF11_HD void stream_group_ragged(uint32_t g, const BlockPlan& p, const uint8_t* stage,
-                                 const uint8_t* sign_mantissa, uint16_t* out) {
+DF11_HD SubSpans spans_of(const SubPlan& p) {
+  SubSpans s;
   const uint32_t first = p.phase, last = p.phase + p.n_out;
+  s.head_begin = first;
+  uint32_t up = (first + (uint32_t)kGroup - 1u) & ~(uint32_t)(kGroup - 1);
+  s.head_end = up < last ? up : last;
+  s.body_begin = s.head_end / (uint32_t)kGroup;       // only meaningful if a body exists
+  s.body_end = last / (uint32_t)kGroup;
+  if (s.body_end < s.body_begin) s.body_end = s.body_begin;
+  const uint32_t body_last = s.body_end * (uint32_t)kGroup;
+  s.tail_begin = body_last > s.head_end ? body_last : s.head_end;
+  s.tail_end = last;
+  return s;
+}
+
+// Body group g: 8 staging bytes + 8 sign|mantissa bytes `m` -> 16 bytes of BF16.
+DF11_HD void stream_group(uint32_t g, const SubPlan& p, const uint8_t* stage, const U32x2& m,
+                          uint16_t* out) {
   const uint32_t s0 = g * (uint32_t)kGroup;
-  const uint32_t lo_i = s0 > first ? s0 : first;
-  const uint32_t hi_i = s0 + (uint32_t)kGroup < last ? s0 + (uint32_t)kGroup : last;
-  for (uint32_t i = lo_i; i < hi_i; ++i) out[p.a0 + i] = merge(stage[i], sign_mantissa[p.a0 + i]);
+  const U32x2 e = load_as<U32x2>(stage + s0);
+  U32x4 o;
+  merge4(e.x, m.x, o.x, o.y);
+  merge4(e.y, m.y, o.z, o.w);
+  store_as<U32x4>(out + p.a0 + s0, o);
+}
+
+// One element of a head or tail (or of everything, for unaligned buffers).
+DF11_HD void stream_element(uint32_t i, const SubPlan& p, const uint8_t* stage,
+                            const uint8_t* sign_mantissa, uint16_t* out) {
+  out[p.a0 + i] = merge(stage[i], sign_mantissa[p.a0 + i]);
 }
 
 }  // namespace df11

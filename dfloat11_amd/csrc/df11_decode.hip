@@ -1,20 +1,20 @@
 // gfx950 kernels and C-ABI for DF11 stream decode.
 //
-// One workgroup of 512 threads (8 wavefronts of 64) handles one 4096-byte
-// bitstream block at a time and walks the grid persistently, so the derived
-// tables are copied into LDS once per workgroup rather than once per block.
-// Per block:
-//   1. every thread takes its 8-byte chunk (+4 bytes of look-ahead) and 5-bit gap
-//      (fetched one block ahead) and counts the codes starting in the chunk with
-//      the four-symbol table in LDS;
-//   2. exclusive prefix sum of the 512 counts: DPP scan inside each wavefront,
-//      eight wavefront totals combined through LDS;
-//   3. every thread decodes its codes again and stores the symbols of each lookup
-//      with one unaligned 32-bit LDS store into a staging area laid out in output
-//      order;
-//   4. the workgroup streams the staging area out: 16 exponent bytes (LDS) + 16
-//      sign|mantissa bytes (global, coalesced, requested before step 1) -> two
-//      16-byte BF16 stores per lane.
+// Unit of work: a sub-block, the 512 bytes of bitstream (64 chunks of 8 bytes)
+// that one 64-lane wavefront decodes.  The output index at which each sub-block
+// starts is derived once per tensor by df11_prepare (it depends only on the
+// compressed stream), so at decode time every wavefront is independent: no
+// workgroup barrier and no exchange between wavefronts, only the decode tables
+// in LDS are shared.  Workgroups of 512 threads walk the sub-blocks persistently
+// (tables are copied into LDS once per workgroup).  Per sub-block a wavefront
+//   1. takes its chunk (+4 bytes of look-ahead), gap and start index, all fetched
+//      one sub-block ahead, and requests the sign|mantissa bytes it will need;
+//   2. counts the codes starting in each lane's chunk (four-symbol table in LDS);
+//   3. turns the 64 counts into exclusive offsets with a DPP scan;
+//   4. decodes again, storing the symbols of each lookup with one unaligned
+//      32-bit store into its private LDS staging area, in output order;
+//   5. streams the staging area out: 8 exponent bytes (LDS) + 8 sign|mantissa
+//      bytes -> one 16-byte BF16 store per lane, contiguous across the wavefront.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -32,28 +32,7 @@ inline int hip_fail(hipError_t e) {
   return DF11_ERR_HIP;
 }
 
-// ---------------------------------------------------------------------------
-// Table builder: one thread per table index.
-// ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void build_tables_kernel(const uint8_t* __restrict__ luts,
-                                                           int n_luts, uint8_t* __restrict__ tables) {
-  const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (uint32_t)kTableEntries) return;
-  // The length row is the last row of `luts`; decode rows beyond the 17 a
-  // pointer can name are unreachable.  Present both as one contiguous view by
-  // staging into LDS: rows [0, n_rows) then the length row.
-  __shared__ uint8_t rows[(kMaxDecodeRows + 1) * 256];
-  const int n_rows = min(n_luts - 1, kMaxDecodeRows);
-  for (int i = threadIdx.x; i < n_rows * 256; i += blockDim.x) rows[i] = luts[i];
-  for (int i = threadIdx.x; i < 256; i += blockDim.x)
-    rows[n_rows * 256 + i] = luts[(n_luts - 1) * 256 + i];
-  __syncthreads();
-  Luts l{rows, n_rows};
-  uint32_t syms, meta;
-  make_dec_entry(l, idx, syms, meta);
-  reinterpret_cast<uint2*>(tables + kDecOffset)[idx] = make_uint2(syms, meta);
-  tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
-}
+constexpr int kWavesPerGroup = kThreads / kLanes;   // 8
 
 // ---------------------------------------------------------------------------
 // Wavefront inclusive scan with DPP (row shifts inside rows of 16 lanes, then
@@ -74,116 +53,235 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
   return v;
 }
 
+__device__ __forceinline__ uint32_t wave_total(uint32_t inclusive) {
+  return (uint32_t)__builtin_amdgcn_readlane((int)inclusive, 63);
+}
+
+// Copies the byte LUT rows a pointer can reach, then the length row, into LDS.
+__device__ __forceinline__ void stage_rows(const uint8_t* __restrict__ luts, int n_luts, int n_rows,
+                                           uint8_t* rows, int tid, int n_threads) {
+  for (int i = tid; i < n_rows * 256; i += n_threads) rows[i] = luts[i];
+  for (int i = tid; i < 256; i += n_threads) rows[n_rows * 256 + i] = luts[(int64_t)(n_luts - 1) * 256 + i];
+}
+
+// ---------------------------------------------------------------------------
+// Prepare, step 1: decode tables + header.  One thread per table index.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void build_tables_kernel(const uint8_t* __restrict__ luts, int n_luts,
+                                                           uint8_t* __restrict__ ws, uint32_t n_blocks) {
+  __shared__ uint8_t rows[(kMaxDecodeRows + 1) * 256];
+  const int n_rows = min(n_luts - 1, kMaxDecodeRows);
+  stage_rows(luts, n_luts, n_rows, rows, threadIdx.x, blockDim.x);
+  __syncthreads();
+  const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (uint32_t)kTableEntries) return;
+  const Luts l{rows, n_rows};
+  uint32_t syms, meta;
+  make_dec_entry(l, idx, syms, meta);
+  uint8_t* tables = ws + kWsTablesOffset;
+  reinterpret_cast<uint2*>(tables + kDecOffset)[idx] = make_uint2(syms, meta);
+  tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
+  if (idx < sizeof(WorkspaceHeader) / 4) {
+    uint32_t v = 0;
+    if (idx == 0) v = kWorkspaceMagic;
+    if (idx == 1) v = n_blocks;
+    reinterpret_cast<uint32_t*>(ws)[idx] = v;   // max_sub_elems starts at 0
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Prepare, step 2: where each sub-block's output starts.  One workgroup per
+// 4096-byte block at a time: count per lane, totals per wavefront, offsets from
+// the block's own output position.
+// ---------------------------------------------------------------------------
+struct IndexArgs {
+  const uint8_t* luts;
+  const uint8_t* codes;
+  const uint32_t* positions;
+  const uint8_t* gaps;
+  uint8_t* ws;
+  int64_t n_bytes;
+  int64_t n_elements;
+  int64_t n_blocks;
+  int32_t n_luts;
+  int32_t codes_aligned;
+};
+
+__global__ __launch_bounds__(kThreads) void index_kernel(const IndexArgs a) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n_rows = min(a.n_luts - 1, kMaxDecodeRows);
+  uint8_t* lds_tables = lds;
+  uint8_t* lds_rows = lds + kTablesBytes;
+  uint32_t* wave_sums = reinterpret_cast<uint32_t*>(lds_rows + (kMaxDecodeRows + 1) * 256);
+  {
+    const uint4* src = reinterpret_cast<const uint4*>(a.ws + kWsTablesOffset);
+    uint4* dst = reinterpret_cast<uint4*>(lds_tables);
+    for (int i = tid; i < kTablesBytes / 16; i += kThreads) dst[i] = src[i];
+    stage_rows(a.luts, a.n_luts, n_rows, lds_rows, tid, kThreads);
+  }
+  __syncthreads();
+  const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
+  const Luts l{lds_rows, n_rows};
+  const int64_t n_gap_bytes = a.n_blocks * kGapBytesPerBlock;
+  uint32_t* subpos = reinterpret_cast<uint32_t*>(a.ws + kWsSubposOffset);
+  uint32_t my_max = 0;
+  for (int64_t blk = blockIdx.x; blk < a.n_blocks; blk += gridDim.x) {
+    const int64_t gid = blk * kThreads + tid;
+    const Chunk c = fetch_chunk(a.codes, a.n_bytes, gid, a.codes_aligned != 0);
+    const uint32_t gap = gap_of(a.gaps, gid, n_gap_bytes);
+    const uint32_t count = count_chunk(t, l, c.hi, c.lo, c.next, gap);
+    const uint32_t incl = wave_inclusive_scan(count);
+    if (lane == 63) wave_sums[wave] = incl;
+    __syncthreads();
+    if (tid < kWavesPerGroup) {
+      int64_t start = (int64_t)a.positions[blk];
+      for (int wv = 0; wv < tid; ++wv) start += wave_sums[wv];
+      int64_t end = start + wave_sums[tid];
+      if (start > a.n_elements) start = a.n_elements;
+      if (end > a.n_elements) end = a.n_elements;
+      subpos[blk * kSubsPerBlock + tid] = (uint32_t)start;
+      my_max = max(my_max, (uint32_t)(end - start));
+    }
+    __syncthreads();   // wave_sums is rewritten by the next block
+  }
+  if (blockIdx.x == 0 && tid == 0) subpos[a.n_blocks * kSubsPerBlock] = (uint32_t)a.n_elements;
+  if (tid < kWavesPerGroup && my_max)
+    atomicMax(&reinterpret_cast<WorkspaceHeader*>(a.ws)->max_sub_elems, my_max);
+}
+
 // ---------------------------------------------------------------------------
 // Decode kernel.
-// LDS layout (dynamic): tables | byte LUT rows + length row | wave sums | stage
+// LDS layout (dynamic): tables | byte LUT rows + length row | 8 staging areas
 // ---------------------------------------------------------------------------
 struct DecodeArgs {
   const uint8_t* luts;
   const uint8_t* codes;
   const uint8_t* sign_mantissa;
-  const uint32_t* positions;
   const uint8_t* gaps;
   uint16_t* out;
-  const uint8_t* tables;
+  const uint8_t* ws;
   int64_t n_bytes;
   int64_t n_elements;
   int64_t n_blocks;
+  int64_t n_subs;         // sub-blocks that hold stream bytes: ceil(n_bytes / 512)
   int32_t n_luts;
-  int32_t stage_cap;      // bytes of staging, multiple of 16
+  int32_t stage_cap;      // bytes of staging per wavefront, multiple of 16
   int32_t codes_aligned;  // codes pointer is 8-byte aligned
-  int32_t vec_ok;         // sign_mantissa and out both 16-byte aligned
+  int32_t vec_ok;         // sign_mantissa 8-byte aligned and out 16-byte aligned
 };
+
+constexpr int kPrefetchGroups = 3;   // body groups per lane whose sign|mantissa bytes are requested early
+
+struct SubInputs {
+  Chunk c;
+  uint32_t gap;
+  uint32_t base;       // first output element
+  uint32_t end_hint;   // first output element of the next sub-block
+};
+
+__device__ __forceinline__ SubInputs fetch_sub(const DecodeArgs& a, const uint32_t* subpos, int64_t sub,
+                                               int lane, int64_t n_gap_bytes) {
+  SubInputs in;
+  const int64_t gid = sub * kLanes + lane;
+  in.c = fetch_chunk(a.codes, a.n_bytes, gid, a.codes_aligned != 0);
+  in.gap = gap_of(a.gaps, gid, n_gap_bytes);
+  in.base = subpos[sub];
+  in.end_hint = subpos[sub + 1];
+  return in;
+}
 
 __global__ __launch_bounds__(kThreads) void decode_kernel(const DecodeArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_rows = min(a.n_luts - 1, kMaxDecodeRows);
   uint8_t* lds_tables = lds;
   uint8_t* lds_rows = lds + kTablesBytes;
-  uint32_t* wave_sums = reinterpret_cast<uint32_t*>(lds_rows + (kMaxDecodeRows + 1) * 256);
-  uint8_t* stage = reinterpret_cast<uint8_t*>(wave_sums + 16);
-
-  // Tables and byte LUTs into LDS, 16 bytes per lane per step.
+  uint8_t* stage = lds_rows + (kMaxDecodeRows + 1) * 256 + (size_t)wave * a.stage_cap;
   {
-    const uint4* src = reinterpret_cast<const uint4*>(a.tables);
+    const uint4* src = reinterpret_cast<const uint4*>(a.ws + kWsTablesOffset);
     uint4* dst = reinterpret_cast<uint4*>(lds_tables);
     for (int i = tid; i < kTablesBytes / 16; i += kThreads) dst[i] = src[i];
-    for (int i = tid; i < n_rows * 256; i += kThreads) lds_rows[i] = a.luts[i];
-    if (tid < 256) lds_rows[n_rows * 256 + tid] = a.luts[(int64_t)(a.n_luts - 1) * 256 + tid];
+    stage_rows(a.luts, a.n_luts, n_rows, lds_rows, tid, kThreads);
   }
-  __syncthreads();
+  __syncthreads();   // the only workgroup barrier: tables are read-only from here on
 
   const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
   const Luts l{lds_rows, n_rows};
   const int64_t n_gap_bytes = a.n_blocks * kGapBytesPerBlock;
+  const uint32_t* subpos = reinterpret_cast<const uint32_t*>(a.ws + kWsSubposOffset);
   const bool vec_ok = a.vec_ok != 0;
+  const int64_t stride = (int64_t)gridDim.x * kWavesPerGroup;
 
-  int64_t blk = blockIdx.x;
-  Chunk c = fetch_chunk(a.codes, a.n_bytes, blk * kThreads + tid, a.codes_aligned != 0);
-  uint32_t gap = gap_of(a.gaps, blk * kThreads + tid, n_gap_bytes);
+  int64_t sub = (int64_t)blockIdx.x * kWavesPerGroup + wave;
+  if (sub >= a.n_subs) return;
+  SubInputs cur = fetch_sub(a, subpos, sub, lane, n_gap_bytes);
 
-  for (; blk < a.n_blocks; blk += gridDim.x) {
-    // ---- requests whose latency the two decode passes hide: the next block's
-    // chunk and gap, and this block's sign|mantissa bytes for the write-out
-    const int64_t next_blk = blk + gridDim.x;
-    Chunk c_next{0, 0, 0};
-    uint32_t gap_next = 0;
-    if (next_blk < a.n_blocks) {
-      c_next = fetch_chunk(a.codes, a.n_bytes, next_blk * kThreads + tid, a.codes_aligned != 0);
-      gap_next = gap_of(a.gaps, next_blk * kThreads + tid, n_gap_bytes);
-    }
-    const int64_t base = (int64_t)a.positions[blk];
+  for (; sub < a.n_subs; sub += stride) {
+    // ---- requests whose latency the two decode passes hide: the next
+    // sub-block's inputs and this one's sign|mantissa bytes
+    const int64_t next_sub = sub + stride;
+    SubInputs nxt = cur;
+    if (next_sub < a.n_subs) nxt = fetch_sub(a, subpos, next_sub, lane, n_gap_bytes);
+
+    const int64_t base = cur.base;
     const int64_t a0 = base & ~(int64_t)(kGroup - 1);
-    U32x4 m0{0, 0, 0, 0}, m1{0, 0, 0, 0};
-    if (vec_ok) {
-      const int64_t i0 = a0 + (int64_t)tid * kGroup, i1 = i0 + (int64_t)kThreads * kGroup;
-      if (i0 + kGroup <= a.n_elements) m0 = load_as<U32x4>(a.sign_mantissa + i0);
-      if (i1 + kGroup <= a.n_elements) m1 = load_as<U32x4>(a.sign_mantissa + i1);
-    }
-
-    // ---- pass 1: how many codes start in my chunk
-    const uint32_t count = count_chunk(t, l, c.hi, c.lo, c.next, gap);
-
-    // ---- exclusive prefix over the workgroup
-    const uint32_t incl = wave_inclusive_scan(count);
-    if (lane == 63) wave_sums[wave] = incl;
-    __syncthreads();
-    uint32_t wave_base = 0, total = 0;
+    int64_t end_hint = cur.end_hint;
+    if (end_hint > a.n_elements) end_hint = a.n_elements;
+    const uint32_t first_body = (base != a0) ? 1u : 0u;   // group 0 is a partial head unless aligned
+    U32x2 m[kPrefetchGroups];
 #pragma unroll
-    for (int wv = 0; wv < kThreads / 64; ++wv) {
-      const uint32_t s = wave_sums[wv];
-      if (wv < wave) wave_base += s;
-      total += s;
+    for (int k = 0; k < kPrefetchGroups; ++k) {
+      m[k] = U32x2{0, 0};
+      const int64_t e0 = a0 + (int64_t)(first_body + lane + kLanes * k) * kGroup;
+      if (vec_ok && e0 + kGroup <= end_hint) m[k] = load_as<U32x2>(a.sign_mantissa + e0);
     }
-    const uint32_t excl = wave_base + incl - count;
 
-    // ---- pass 2: decode into the staging area, in output order
-    const BlockPlan p = plan_block(base, total, a.n_elements, a.stage_cap);
-    emit_chunk(t, l, c.hi, c.lo, c.next, gap, thread_quota(excl, count, p.n_out),
+    // ---- pass 1 and the exclusive offsets inside the wavefront
+    const uint32_t count = count_chunk(t, l, cur.c.hi, cur.c.lo, cur.c.next, cur.gap);
+    const uint32_t incl = wave_inclusive_scan(count);
+    const uint32_t total = wave_total(incl);
+    const uint32_t excl = incl - count;
+
+    // ---- pass 2: decode into this wavefront's staging area, in output order
+    const SubPlan p = plan_sub(base, total, a.n_elements, a.stage_cap);
+    emit_chunk(t, l, cur.c.hi, cur.c.lo, cur.c.next, cur.gap, thread_quota(excl, count, p.n_out),
                stage + p.phase + excl);
-    __syncthreads();
+    // Staging is exchanged between the lanes of one wavefront only; its LDS
+    // operations execute in order, the fence keeps the compiler from reordering.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-    // ---- stream out, 16 elements per lane per step.  No barrier is needed after
-    // this: the next block's staging writes come after its prefix-sum barrier,
-    // which every wavefront reaches only when it is done reading here.
-    const uint32_t n_groups = n_groups_of(p);
-    for (uint32_t g = tid; g < n_groups; g += kThreads) {
-      if (vec_ok && group_is_full(g, p)) {
-        U32x4 m;
-        if (g == (uint32_t)tid) m = m0;
-        else if (g == (uint32_t)(tid + kThreads)) m = m1;
-        else m = load_as<U32x4>(a.sign_mantissa + p.a0 + (int64_t)g * kGroup);
-        stream_group_full(g, p, stage, m, a.out);
-      } else {
-        stream_group_ragged(g, p, stage, a.sign_mantissa, a.out);
+    // ---- stream out
+    const SubSpans sp = spans_of(p);
+    if (vec_ok) {
+      for (uint32_t i = sp.head_begin + lane; i < sp.head_end; i += kLanes)
+        stream_element(i, p, stage, a.sign_mantissa, a.out);
+      uint32_t g = sp.body_begin + lane;
+#pragma unroll
+      for (int k = 0; k < kPrefetchGroups; ++k, g += kLanes) {
+        if (g < sp.body_end) {
+          // requested early only when the hint covered the group; the hint is the
+          // next sub-block's start, which equals this one's end for a valid stream
+          const int64_t e0 = p.a0 + (int64_t)g * kGroup;
+          const bool early = sp.body_begin == first_body && e0 + kGroup <= end_hint;
+          const U32x2 mm = early ? m[k] : load_as<U32x2>(a.sign_mantissa + e0);
+          stream_group(g, p, stage, mm, a.out);
+        }
       }
+      for (; g < sp.body_end; g += kLanes)
+        stream_group(g, p, stage, load_as<U32x2>(a.sign_mantissa + p.a0 + (int64_t)g * kGroup), a.out);
+      for (uint32_t i = sp.tail_begin + lane; i < sp.tail_end; i += kLanes)
+        stream_element(i, p, stage, a.sign_mantissa, a.out);
+    } else {
+      for (uint32_t i = p.phase + lane; i < p.phase + p.n_out; i += kLanes)
+        stream_element(i, p, stage, a.sign_mantissa, a.out);
     }
-    c = c_next;
-    gap = gap_next;
+    // The next sub-block's staging stores must not pass this one's loads.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    cur = nxt;
   }
 }
 
@@ -218,13 +316,20 @@ int device_info(DeviceInfo& info) {
   return DF11_OK;
 }
 
-constexpr int kFixedLds = kTablesBytes + (kMaxDecodeRows + 1) * 256 + 16 * 4;
+constexpr int kFixedLds = kTablesBytes + (kMaxDecodeRows + 1) * 256;
+constexpr int kLdsPerCu = 160 * 1024;
+
+int groups_per_cu(size_t lds_bytes) {
+  int n = (int)(kLdsPerCu / lds_bytes);
+  if (n > 4) n = 4;     // 2048 threads per CU
+  return n < 1 ? 1 : n;
+}
 
 }  // namespace
 
 extern "C" {
 
-int df11_version(void) { return 1; }
+int df11_version(void) { return 2; }
 
 const char* df11_error_string(int code) {
   switch (code) {
@@ -240,16 +345,59 @@ const char* df11_error_string(int code) {
 
 const char* df11_last_hip_error(void) { return hipGetErrorString(g_last_hip); }
 
-size_t df11_tables_bytes(void) { return kTablesBytes; }
+size_t df11_workspace_bytes(int64_t n_bytes) {
+  if (n_bytes < 0) return 0;
+  return (size_t)workspace_bytes((n_bytes + kBlockBytes - 1) / kBlockBytes);
+}
 
-int df11_build_tables(const uint8_t* luts, int32_t n_luts, void* tables, void* stream) {
-  if (!luts || !tables || n_luts < 2) return DF11_ERR_INVALID_ARGUMENT;
-  if (reinterpret_cast<uintptr_t>(tables) & 15) return DF11_ERR_INVALID_ARGUMENT;
-  hipLaunchKernelGGL(build_tables_kernel, dim3(kTableEntries / 256), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), luts, (int)n_luts,
-                     static_cast<uint8_t*>(tables));
+int df11_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const uint32_t* output_positions,
+                 const uint8_t* gaps, int32_t n_luts, int64_t n_bytes, int64_t n_elements,
+                 void* workspace, int32_t* max_elems_per_subblock, void* stream) {
+  if (n_bytes < 0 || n_elements < 0 || n_luts < 2 || !luts || !workspace) return DF11_ERR_INVALID_ARGUMENT;
+  if (n_elements >= ((int64_t)1 << 32)) return DF11_ERR_UNSUPPORTED;   // positions are u32
+  if (n_bytes > 0 && (!encoded_exponent || !output_positions || !gaps)) return DF11_ERR_INVALID_ARGUMENT;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 15) || (reinterpret_cast<uintptr_t>(output_positions) & 3))
+    return DF11_ERR_INVALID_ARGUMENT;
+  DeviceInfo info;
+  if (int rc = device_info(info)) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  if (n_blocks >= ((int64_t)1 << 28)) return DF11_ERR_UNSUPPORTED;
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+
+  hipLaunchKernelGGL(build_tables_kernel, dim3(kTableEntries / 256), dim3(256), 0, s, luts, (int)n_luts,
+                     ws, (uint32_t)n_blocks);
   hipError_t e = hipGetLastError();
-  return e == hipSuccess ? DF11_OK : hip_fail(e);
+  if (e != hipSuccess) return hip_fail(e);
+
+  if (n_blocks > 0) {
+    IndexArgs a;
+    a.luts = luts;
+    a.codes = encoded_exponent;
+    a.positions = output_positions;
+    a.gaps = gaps;
+    a.ws = ws;
+    a.n_bytes = n_bytes;
+    a.n_elements = n_elements;
+    a.n_blocks = n_blocks;
+    a.n_luts = n_luts;
+    a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
+    const size_t lds_bytes = (size_t)kFixedLds + 64;
+    int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
+    if (grid > n_blocks) grid = n_blocks;
+    hipLaunchKernelGGL(index_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+  }
+  if (max_elems_per_subblock) {
+    WorkspaceHeader h;
+    e = hipMemcpyAsync(&h, ws, sizeof h, hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return hip_fail(e);
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(e);
+    *max_elems_per_subblock = (int32_t)h.max_sub_elems;
+  }
+  return DF11_OK;
 }
 
 int df11_calibration_copy(const void* src, void* dst, int64_t n_bytes, void* stream) {
@@ -267,17 +415,17 @@ int df11_calibration_copy(const void* src, void* dst, int64_t n_bytes, void* str
 
 int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
                 const uint32_t* output_positions, const uint8_t* gaps, uint16_t* outputs,
-                int32_t n_luts, int64_t n_bytes, int64_t n_elements, int32_t max_elems_per_block,
-                const void* tables, void* stream) {
+                int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void* workspace,
+                int32_t max_elems_per_subblock, void* stream) {
+  (void)output_positions;   // superseded by the sub-block positions in the workspace
   if (n_bytes < 0 || n_elements < 0 || n_luts < 2) return DF11_ERR_INVALID_ARGUMENT;
   if (n_bytes == 0 || n_elements == 0) return DF11_OK;
-  if (!luts || !encoded_exponent || !sign_mantissa || !output_positions || !gaps || !outputs || !tables)
+  if (!luts || !encoded_exponent || !sign_mantissa || !gaps || !outputs || !workspace)
     return DF11_ERR_INVALID_ARGUMENT;
-  if ((reinterpret_cast<uintptr_t>(tables) & 15) || (reinterpret_cast<uintptr_t>(outputs) & 1) ||
-      (reinterpret_cast<uintptr_t>(output_positions) & 3))
+  if ((reinterpret_cast<uintptr_t>(workspace) & 15) || (reinterpret_cast<uintptr_t>(outputs) & 1))
     return DF11_ERR_INVALID_ARGUMENT;
-  if (max_elems_per_block <= 0 || max_elems_per_block > kMaxElemsPerBlock)
-    max_elems_per_block = kMaxElemsPerBlock;
+  if (max_elems_per_subblock <= 0 || max_elems_per_subblock > kMaxElemsPerSub)
+    max_elems_per_subblock = kMaxElemsPerSub;
 
   DeviceInfo info;
   if (int rc = device_info(info)) return rc;
@@ -286,25 +434,23 @@ int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint
   a.luts = luts;
   a.codes = encoded_exponent;
   a.sign_mantissa = sign_mantissa;
-  a.positions = output_positions;
   a.gaps = gaps;
   a.out = outputs;
-  a.tables = static_cast<const uint8_t*>(tables);
+  a.ws = static_cast<const uint8_t*>(workspace);
   a.n_bytes = n_bytes;
   a.n_elements = n_elements;
   a.n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  a.n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
   a.n_luts = n_luts;
-  a.stage_cap = ((max_elems_per_block + kGroup + 15) / 16) * 16;   // + up to 15 elements of output phase
+  a.stage_cap = ((max_elems_per_subblock + kGroup + 15) / 16) * 16;   // + up to 7 elements of output phase
   a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
-  a.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 15) == 0 &&
+  a.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
              (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
 
-  const size_t lds_bytes = (size_t)kFixedLds + (size_t)a.stage_cap;
-  int wgs_per_cu = (int)((160 * 1024) / lds_bytes);
-  if (wgs_per_cu > 4) wgs_per_cu = 4;     // 2048 threads per CU
-  if (wgs_per_cu < 1) wgs_per_cu = 1;
-  int64_t grid = (int64_t)info.cus * wgs_per_cu;
-  if (grid > a.n_blocks) grid = a.n_blocks;
+  const size_t lds_bytes = (size_t)kFixedLds + (size_t)kWavesPerGroup * (size_t)a.stage_cap;
+  int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
+  const int64_t needed = (a.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
+  if (grid > needed) grid = needed;
 
   hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes,
                      static_cast<hipStream_t>(stream), a);

@@ -21,45 +21,61 @@ def _require_cuda(**tensors):
             raise _native.DF11Error(f"{name} must be contiguous")
 
 
-def tables_bytes():
-    return int(_native.hip_lib().df11_tables_bytes())
+def workspace_bytes(n_bytes):
+    return int(_native.hip_lib().df11_workspace_bytes(int(n_bytes)))
 
 
-def build_tables(luts, out=None):
-    """Derive the multi-symbol decode tables for `luts` (u8 [n_luts, 256], on the GPU)."""
-    _require_cuda(luts=luts)
+def _check_stream_tensors(luts, encoded_exponent, output_positions, gaps):
     if luts.dtype != torch.uint8 or luts.dim() != 2 or luts.shape[1] != 256 or luts.shape[0] < 2:
         raise _native.DF11Error(f"luts must be uint8 [n_luts >= 2, 256], got {luts.dtype} {tuple(luts.shape)}")
-    if out is None:
-        out = torch.empty(tables_bytes(), dtype=torch.uint8, device=luts.device)
-    with torch.cuda.device(luts.device):
-        rc = _native.hip_lib().df11_build_tables(luts.data_ptr(), luts.shape[0], out.data_ptr(),
-                                                 _stream_ptr(luts.device))
-    _native.check(rc, "df11_build_tables")
-    return out
-
-
-def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, tables,
-           max_elems_per_block=0):
-    """Decode one DF11 stream into `out` (bfloat16, >= n_elements) on the current stream."""
-    _require_cuda(luts=luts, encoded_exponent=encoded_exponent, sign_mantissa=sign_mantissa,
-                  output_positions=output_positions, gaps=gaps, out=out, tables=tables)
-    n_elements = sign_mantissa.numel()
-    n_bytes = encoded_exponent.numel()
-    n_blocks = -(-n_bytes // 4096)
-    if out.dtype != torch.bfloat16 or out.numel() < n_elements:
-        raise _native.DF11Error("out must be a bfloat16 tensor with at least n_elements elements")
+    n_blocks = -(-encoded_exponent.numel() // 4096)
     if output_positions.numel() * output_positions.element_size() < 4 * n_blocks:
         raise _native.DF11Error("output_positions shorter than one entry per bitstream block")
     if gaps.numel() < 320 * n_blocks:
         raise _native.DF11Error("gaps shorter than 320 bytes per bitstream block")
-    if tables.numel() * tables.element_size() < tables_bytes():
-        raise _native.DF11Error("tables buffer too small")
+
+
+def prepare(luts, encoded_exponent, output_positions, gaps, n_elements, workspace=None):
+    """Build the decode workspace of one stream (load time; waits for the current stream).
+    Returns (workspace uint8 tensor, max_elems_per_subblock)."""
+    import ctypes
+    _require_cuda(luts=luts, encoded_exponent=encoded_exponent, output_positions=output_positions, gaps=gaps)
+    _check_stream_tensors(luts, encoded_exponent, output_positions, gaps)
+    n_bytes = encoded_exponent.numel()
+    need = workspace_bytes(n_bytes)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=luts.device)
+    else:
+        _require_cuda(workspace=workspace)
+        if workspace.numel() * workspace.element_size() < need:
+            raise _native.DF11Error("workspace buffer too small")
+    max_sub = ctypes.c_int32(0)
+    with torch.cuda.device(luts.device):
+        rc = _native.hip_lib().df11_prepare(
+            luts.data_ptr(), encoded_exponent.data_ptr(), output_positions.data_ptr(), gaps.data_ptr(),
+            luts.shape[0], n_bytes, int(n_elements), workspace.data_ptr(), ctypes.byref(max_sub),
+            _stream_ptr(luts.device))
+    _native.check(rc, "df11_prepare")
+    return workspace, int(max_sub.value)
+
+
+def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,
+           max_elems_per_subblock=0):
+    """Decode one DF11 stream into `out` (bfloat16, >= n_elements) on the current stream."""
+    _require_cuda(luts=luts, encoded_exponent=encoded_exponent, sign_mantissa=sign_mantissa,
+                  output_positions=output_positions, gaps=gaps, out=out, workspace=workspace)
+    _check_stream_tensors(luts, encoded_exponent, output_positions, gaps)
+    n_elements = sign_mantissa.numel()
+    n_bytes = encoded_exponent.numel()
+    if out.dtype != torch.bfloat16 or out.numel() < n_elements:
+        raise _native.DF11Error("out must be a bfloat16 tensor with at least n_elements elements")
+    if workspace.numel() * workspace.element_size() < workspace_bytes(n_bytes):
+        raise _native.DF11Error("workspace buffer too small")
     with torch.cuda.device(out.device):
         rc = _native.hip_lib().df11_decode(
             luts.data_ptr(), encoded_exponent.data_ptr(), sign_mantissa.data_ptr(),
             output_positions.data_ptr(), gaps.data_ptr(), out.data_ptr(),
-            luts.shape[0], n_bytes, n_elements, int(max_elems_per_block), tables.data_ptr(),
+            luts.shape[0], n_bytes, n_elements, workspace.data_ptr(), int(max_elems_per_subblock),
             _stream_ptr(out.device))
     _native.check(rc, "df11_decode")
     return out

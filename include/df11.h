@@ -7,8 +7,9 @@
  *
  * Conventions: every function returns DF11_OK (0) or a negative DF11_ERR_*
  * code; df11_error_string() names it.  The library never allocates or frees
- * device memory and never synchronises the device: kernels are enqueued on the
- * caller's stream and the caller owns every buffer until that work completes.
+ * device memory: kernels are enqueued on the caller's stream and the caller owns
+ * every buffer until that work completes.  Only df11_prepare (load time) may
+ * wait for the stream; df11_decode never synchronises.
  * `stream` is a hipStream_t passed as void* (NULL = the default stream).
  */
 #ifndef DF11_H
@@ -34,6 +35,8 @@ extern "C" {
 #define DF11_BLOCK_BYTES 4096
 #define DF11_GAP_BYTES_PER_BLOCK 320
 #define DF11_MAX_ELEMS_PER_BLOCK 32768
+#define DF11_SUBBLOCK_BYTES 512
+#define DF11_MAX_ELEMS_PER_SUBBLOCK 4096
 
 int df11_version(void);
 const char *df11_error_string(int code);
@@ -44,20 +47,28 @@ const char *df11_error_string(int code);
 const char *df11_last_hip_error(void);
 
 /*
- * Size in bytes of the derived decode tables for one compressed tensor.
- * The tables depend only on `luts`; build them once per tensor (at load time)
- * and keep them next to it.  No counterpart in the reference, whose kernel
- * chases the byte LUTs in global memory on every symbol (decode.cu:105-116).
+ * Size in bytes of the decode workspace of a stream with n_bytes bytes of
+ * encoded_exponent: a 64-byte header, the multi-symbol decode tables derived
+ * from `luts`, and the output index at which each 512-byte sub-block of the
+ * bitstream starts (4 bytes per sub-block, about 0.2 % of the compressed size).
  */
-size_t df11_tables_bytes(void);
+size_t df11_workspace_bytes(int64_t n_bytes);
 
 /*
- * Derive the multi-symbol decode tables from the DF11 byte LUTs.
- *   luts    device, u8[n_luts][256]: rows 0..n_luts-2 hierarchical decode LUTs,
- *           row n_luts-1 code lengths (layout: dfloat11_utils.py:68-115)
- *   tables  device, df11_tables_bytes() bytes, 16-byte aligned
+ * Fill the workspace of one compressed tensor.  Everything in it depends only on
+ * the compressed stream, so this runs once per tensor at load time; the
+ * reference's closest counterpart is the load-time derivation of shared_mem_size
+ * from output_positions (dfloat11/dfloat11.py:299-306).
+ *   luts, encoded_exponent, output_positions, gaps   as for df11_decode (device)
+ *   workspace   device, df11_workspace_bytes(n_bytes) bytes, 16-byte aligned
+ *   max_elems_per_subblock   host out, may be NULL: the largest number of
+ *               elements any 512-byte sub-block produces; pass it to df11_decode.
+ *               When non-NULL the call waits for `stream` (load time only).
  */
-int df11_build_tables(const uint8_t *luts, int32_t n_luts, void *tables, void *stream);
+int df11_prepare(const uint8_t *luts, const uint8_t *encoded_exponent,
+                 const uint32_t *output_positions, const uint8_t *gaps,
+                 int32_t n_luts, int64_t n_bytes, int64_t n_elements,
+                 void *workspace, int32_t *max_elems_per_subblock, void *stream);
 
 /*
  * Decode one DF11 stream into BF16.  Replaces the reference's kernel launch
@@ -65,19 +76,20 @@ int df11_build_tables(const uint8_t *luts, int32_t n_luts, void *tables, void *s
  *           output_positions, gaps, reconstructed, n_luts, n_bytes, n_elements])
  * (dfloat11/dfloat11.py:139-151; kernel signature dfloat11/decode.cu:25-34).
  * The six pointers and three sizes keep the reference's order and meaning;
- * sizes are 64-bit here.  All pointers are device pointers.
- *   output_positions  u32[ceil(n_bytes/4096)] at least (the entry after the
- *                     last block is not read)
+ * sizes are 64-bit here.  All pointers are device pointers.  Asynchronous on
+ * `stream`; allocates nothing.
+ *   output_positions  u32[ceil(n_bytes/4096)] at least; only df11_prepare reads
+ *                     it, the decode uses the finer positions in the workspace
  *   gaps              u8[320 * ceil(n_bytes/4096)]
- *   max_elems_per_block  max(diff(output_positions)), what the reference keeps
- *                     as (shared_mem_size - 2052) / 2 (dfloat11.py:301-306);
- *                     <= 0 selects the format's worst case (32768)
- *   tables            from df11_build_tables() for the same luts
+ *   workspace         filled by df11_prepare for the same stream
+ *   max_elems_per_subblock  as returned by df11_prepare (it sizes the LDS
+ *                     staging, the role shared_mem_size plays in the reference);
+ *                     <= 0 selects the format's worst case (4096)
  */
 int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint8_t *sign_mantissa,
                 const uint32_t *output_positions, const uint8_t *gaps, uint16_t *outputs,
                 int32_t n_luts, int64_t n_bytes, int64_t n_elements,
-                int32_t max_elems_per_block, const void *tables, void *stream);
+                const void *workspace, int32_t max_elems_per_subblock, void *stream);
 
 /*
  * Streaming device copy of n_bytes (multiple of 16, both pointers 16-byte

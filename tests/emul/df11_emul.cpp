@@ -40,17 +40,61 @@ extern "C" int df11_emul_tables(const uint8_t* luts, int n_luts, uint8_t* tables
   return 0;
 }
 
-// Same arguments as df11_decode (include/df11.h), host pointers; `grid` plays
-// gridDim.x.  n_positions/n_gap_bytes/out_elems size the bounds-checked copies.
+// Host counterpart of df11_prepare: header, tables and the start index of every
+// sub-block.  `ws` has workspace_bytes(n_blocks) bytes.  Returns the largest
+// number of elements a sub-block produces.
+extern "C" int df11_emul_prepare(const uint8_t* luts, const uint8_t* codes, const uint32_t* positions,
+                                 const uint8_t* gaps, int n_luts, int64_t n_bytes, int64_t n_elements,
+                                 uint8_t* ws) {
+  const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
+  memset(ws, 0, (size_t)workspace_bytes(n_blocks));
+  df11_emul_tables(luts, n_luts, ws + kWsTablesOffset);
+  std::vector<uint8_t> rows((size_t)(n_rows + 1) * 256);
+  memcpy(rows.data(), luts, (size_t)n_rows * 256);
+  memcpy(rows.data() + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
+  const Tables t{ws + kWsTablesOffset + kDecOffset, ws + kWsTablesOffset + kCntTailOffset};
+  const Luts l{rows.data(), n_rows};
+  std::vector<uint32_t> subpos((size_t)n_blocks * kSubsPerBlock + 1);
+  uint32_t max_sub = 0;
+  for (int64_t blk = 0; blk < n_blocks; ++blk) {
+    int64_t start = positions[blk];
+    for (int w = 0; w < kSubsPerBlock; ++w) {
+      uint32_t total = 0;
+      for (int lane = 0; lane < kLanes; ++lane) {
+        const int64_t gid = (blk * kSubsPerBlock + w) * kLanes + lane;
+        const Chunk c = fetch_chunk(codes, n_bytes, gid, false);
+        total += count_chunk(t, l, c.hi, c.lo, c.next, gap_of(gaps, gid, n_blocks * kGapBytesPerBlock));
+      }
+      int64_t s0 = start < n_elements ? start : n_elements;
+      int64_t e0 = start + total < n_elements ? start + total : n_elements;
+      subpos[(size_t)(blk * kSubsPerBlock + w)] = (uint32_t)s0;
+      if ((uint32_t)(e0 - s0) > max_sub) max_sub = (uint32_t)(e0 - s0);
+      start += total;
+    }
+  }
+  subpos[(size_t)n_blocks * kSubsPerBlock] = (uint32_t)n_elements;
+  memcpy(ws + kWsSubposOffset, subpos.data(), subpos.size() * 4);
+  WorkspaceHeader h{};
+  h.magic = kWorkspaceMagic;
+  h.n_blocks = (uint32_t)n_blocks;
+  h.max_sub_elems = max_sub;
+  memcpy(ws, &h, sizeof h);
+  return (int)max_sub;
+}
+
+// Same data arguments as df11_decode (include/df11.h), host pointers; `grid`
+// plays gridDim.x (workgroups of eight wavefronts).  max_elems_per_sub <= 0
+// selects the worst case, as in the library.
 extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
                                 const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
                                 int n_luts, int64_t n_bytes, int64_t n_elements,
-                                int max_elems_per_block, int grid, int codes_misalign,
+                                int max_elems_per_sub, int grid, int codes_misalign,
                                 int out_misalign) {
-  if (max_elems_per_block <= 0 || max_elems_per_block > kMaxElemsPerBlock)
-    max_elems_per_block = kMaxElemsPerBlock;
+  if (max_elems_per_sub <= 0 || max_elems_per_sub > kMaxElemsPerSub) max_elems_per_sub = kMaxElemsPerSub;
   const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
-  const int stage_cap = ((max_elems_per_block + kGroup + 15) / 16) * 16;
+  const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
+  const int stage_cap = ((max_elems_per_sub + kGroup + 15) / 16) * 16;
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
 
   // exact-size copies of everything the kernel may read
@@ -67,57 +111,56 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   Exact<uint16_t> c_out((size_t)n_elements + out_misalign);
   uint16_t* out_p = c_out.p + out_misalign;
   memset(c_out.p, 0xEE, ((size_t)n_elements + out_misalign) * 2);
-  Exact<uint8_t> tables((size_t)kTablesBytes);
-  df11_emul_tables(luts, n_luts, tables.p);
+  Exact<uint8_t> ws((size_t)workspace_bytes(n_blocks));
+  df11_emul_prepare(luts, codes_p, c_pos.p, c_gaps.p, n_luts, n_bytes, n_elements, ws.p);
   Exact<uint8_t> rows((size_t)(n_rows + 1) * 256);
   memcpy(rows.p, luts, (size_t)n_rows * 256);
   memcpy(rows.p + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
   Exact<uint8_t> stage((size_t)stage_cap);
 
-  const Tables t{tables.p + kDecOffset, tables.p + kCntTailOffset};
+  const Tables t{ws.p + kWsTablesOffset + kDecOffset, ws.p + kWsTablesOffset + kCntTailOffset};
   const Luts l{rows.p, n_rows};
+  const uint32_t* subpos = reinterpret_cast<const uint32_t*>(ws.p + kWsSubposOffset);
   const bool codes_aligned = (reinterpret_cast<uintptr_t>(codes_p) & 7) == 0;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(sm_p) & 15) == 0 &&
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(sm_p) & 7) == 0 &&
                       (reinterpret_cast<uintptr_t>(out_p) & 15) == 0;
   const int64_t n_gap_bytes = n_blocks * kGapBytesPerBlock;
+  const int64_t stride = (int64_t)grid * kSubsPerBlock;
 
-  std::vector<Chunk> chunk(kThreads);
-  std::vector<uint32_t> gap(kThreads), count(kThreads);
-  for (int wg = 0; wg < grid; ++wg) {
-    for (int64_t blk = wg; blk < n_blocks; blk += grid) {
+  std::vector<Chunk> chunk(kLanes);
+  std::vector<uint32_t> gap(kLanes), count(kLanes), excl(kLanes);
+  for (int64_t wave_gid = 0; wave_gid < stride; ++wave_gid) {
+    for (int64_t sub = wave_gid; sub < n_subs; sub += stride) {
       uint32_t total = 0;
-      for (int tid = 0; tid < kThreads; ++tid) {
-        const int64_t gid = blk * kThreads + tid;
-        chunk[tid] = fetch_chunk(codes_p, n_bytes, gid, codes_aligned);
-        gap[tid] = gap_of(c_gaps.p, gid, n_gap_bytes);
-        count[tid] = count_chunk(t, l, chunk[tid].hi, chunk[tid].lo, chunk[tid].next, gap[tid]);
-        total += count[tid];
+      for (int lane = 0; lane < kLanes; ++lane) {
+        const int64_t gid = sub * kLanes + lane;
+        chunk[lane] = fetch_chunk(codes_p, n_bytes, gid, codes_aligned);
+        gap[lane] = gap_of(c_gaps.p, gid, n_gap_bytes);
+        count[lane] = count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
+        excl[lane] = total;
+        total += count[lane];
       }
-      const BlockPlan p = plan_block((int64_t)c_pos.p[blk], total, n_elements, stage_cap);
+      const SubPlan p = plan_sub((int64_t)subpos[sub], total, n_elements, stage_cap);
       memset(stage.p, 0xDD, (size_t)stage_cap);
-      // Threads of a block run concurrently on the device, so no thread may rely
-      // on a later thread repairing what it wrote.  Even blocks emit in ascending
-      // thread order, odd blocks in descending order: a store that strays into a
-      // neighbour's bytes corrupts the result in one of the two.
-      std::vector<uint32_t> excl(kThreads);
-      uint32_t run = 0;
-      for (int tid = 0; tid < kThreads; ++tid) {
-        excl[tid] = run;
-        run += count[tid];
+      // Lanes run concurrently on the device, so no lane may rely on a later lane
+      // repairing what it wrote.  Even sub-blocks emit in ascending lane order,
+      // odd ones in descending order: a store that strays into a neighbour's
+      // bytes corrupts the result in one of the two.
+      for (int k = 0; k < kLanes; ++k) {
+        const int lane = (sub & 1) ? kLanes - 1 - k : k;
+        const uint32_t quota = thread_quota(excl[lane], count[lane], p.n_out);
+        // a lane with nothing to write may hold an out-of-range pointer; it must not use it
+        emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota,
+                   quota ? stage.p + p.phase + excl[lane] : nullptr);
       }
-      for (int k = 0; k < kThreads; ++k) {
-        const int tid = (blk & 1) ? kThreads - 1 - k : k;
-        const uint32_t quota = thread_quota(excl[tid], count[tid], p.n_out);
-        // a thread with nothing to write may hold an out-of-range pointer; it must not use it
-        emit_chunk(t, l, chunk[tid].hi, chunk[tid].lo, chunk[tid].next, gap[tid], quota,
-                   quota ? stage.p + p.phase + excl[tid] : nullptr);
-      }
-      const uint32_t n_groups = n_groups_of(p);
-      for (uint32_t g = 0; g < n_groups; ++g) {
-        if (vec_ok && group_is_full(g, p))
-          stream_group_full(g, p, stage.p, load_as<U32x4>(sm_p + p.a0 + (int64_t)g * kGroup), out_p);
-        else
-          stream_group_ragged(g, p, stage.p, sm_p, out_p);
+      const SubSpans sp = spans_of(p);
+      if (vec_ok) {
+        for (uint32_t i = sp.head_begin; i < sp.head_end; ++i) stream_element(i, p, stage.p, sm_p, out_p);
+        for (uint32_t g = sp.body_begin; g < sp.body_end; ++g)
+          stream_group(g, p, stage.p, load_as<U32x2>(sm_p + p.a0 + (int64_t)g * kGroup), out_p);
+        for (uint32_t i = sp.tail_begin; i < sp.tail_end; ++i) stream_element(i, p, stage.p, sm_p, out_p);
+      } else {
+        for (uint32_t i = p.phase; i < p.phase + p.n_out; ++i) stream_element(i, p, stage.p, sm_p, out_p);
       }
     }
   }

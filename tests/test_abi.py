@@ -25,20 +25,22 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_error_strings():
     hip = _native.hip_lib()
-    assert hip.df11_version() == 1
+    assert hip.df11_version() == 2
     assert hip.df11_error_string(0) == b"ok"
     assert hip.df11_error_string(-1) == b"invalid argument"
-    assert hip.df11_tables_bytes() == 2048 * 8 + 2048
+    # header + tables + (8 sub-blocks per 4096-byte block + 1) positions, rounded to 16
+    assert hip.df11_workspace_bytes(0) == 64 + 2048 * 8 + 2048 + 16
+    assert hip.df11_workspace_bytes(4097) == 64 + 2048 * 8 + 2048 + ((4 * 17 + 15) // 16) * 16
 
 
 def test_argument_validation_needs_no_gpu():
     hip = _native.hip_lib()
     # null pointers / bad sizes are rejected before any HIP call
-    assert hip.df11_build_tables(None, 4, None, None) == -1
-    assert hip.df11_decode(None, None, None, None, None, None, 4, 100, 100, 0, None, None) == -1
-    assert hip.df11_decode(None, None, None, None, None, None, 4, -1, 100, 0, None, None) == -1
+    assert hip.df11_prepare(None, None, None, None, 4, 100, 100, None, None, None) == -1
+    assert hip.df11_decode(None, None, None, None, None, None, 4, 100, 100, None, 0, None) == -1
+    assert hip.df11_decode(None, None, None, None, None, None, 4, -1, 100, None, 0, None) == -1
     # empty streams decode to nothing
-    assert hip.df11_decode(None, None, None, None, None, None, 4, 0, 0, 0, None, None) == 0
+    assert hip.df11_decode(None, None, None, None, None, None, 4, 0, 0, None, 0, None) == 0
 
 
 def test_decode_without_gpu_fails_loudly():
@@ -48,8 +50,9 @@ def test_decode_without_gpu_fails_loudly():
     if torch.cuda.is_available():
         pytest.skip("GPU present")
     t = torch.zeros(2, 256, dtype=torch.uint8)
+    e = torch.zeros(16, dtype=torch.uint8)
     with pytest.raises(_native.DF11Error):
-        decode.build_tables(t)
+        decode.prepare(t, e, e, e, 4)
 
 
 def test_libraries_are_in_tree():

@@ -32,13 +32,14 @@ def to_gpu(c, pad_front=0):
 def gpu_decode(c, max_elems=None, pad_front=0, out=None):
     g = to_gpu(c, pad_front)
     n = c["sign_mantissa"].size
-    tables = D.build_tables(g["luts"].contiguous())
+    ws, max_sub = D.prepare(g["luts"].contiguous(), g["encoded_exponent"], g["output_positions"],
+                            g["gaps"], n)
     if out is None:
         out = torch.full((n,), float("nan"), dtype=torch.bfloat16, device=DEV)
     if max_elems is None:
-        max_elems = max_elems_per_block(c["output_positions"])
+        max_elems = max_sub
     D.decode(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
-             out, tables, max_elems)
+             out, ws, max_elems)
     torch.cuda.synchronize()
     return out.view(torch.int16).cpu().numpy().view(np.uint16)[:n]
 
@@ -64,22 +65,31 @@ def test_gpu_worst_case_staging(kind):
     assert np.array_equal(gpu_decode(c, max_elems=0), w)
 
 
-def test_gpu_tables_match_host_build():
-    print("case tables", flush=True)
+def test_gpu_workspace_matches_host_build():
+    """Header, tables and sub-block positions: device build == host build of the same code."""
+    print("case workspace", flush=True)
     emul_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
     lib_path = os.path.join(emul_dir, "libdf11_emul.so")
     if not os.path.exists(lib_path):
         subprocess.run(["make", "-s", "-C", emul_dir, "libdf11_emul.so"], check=True)
     L = ctypes.CDLL(lib_path)
-    for kind in ("normal", "fib", "uniform256", "high"):
-        c = compress_product(make_case(kind, 400_000, 71))
+    vp = ctypes.c_void_p
+    L.df11_emul_prepare.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, vp]
+    for kind, n in (("normal", 400_000), ("fib", 400_000), ("uniform256", 100_000), ("high", 9_000),
+                    ("zeros", 300_000), ("single", 5)):
+        c = compress_product(make_case(kind, n, 71))
         luts = np.ascontiguousarray(c["luts"])
-        host = np.zeros(D.tables_bytes(), np.uint8)
-        L.df11_emul_tables(luts.ctypes.data_as(ctypes.c_void_p), luts.shape[0],
-                           host.ctypes.data_as(ctypes.c_void_p))
-        dev = D.build_tables(torch.from_numpy(luts).to(DEV))
+        host = np.zeros(D.workspace_bytes(c["encoded_exponent"].size), np.uint8)
+        p = lambda a: a.ctypes.data_as(vp)
+        host_max = L.df11_emul_prepare(p(luts), p(c["encoded_exponent"]), p(c["output_positions"]),
+                                       p(c["gaps"]), luts.shape[0], c["encoded_exponent"].size, n, p(host))
+        g = to_gpu(c)
+        dev, dev_max = D.prepare(g["luts"], g["encoded_exponent"], g["output_positions"], g["gaps"], n)
         torch.cuda.synchronize()
-        assert np.array_equal(dev.cpu().numpy(), host), kind
+        assert dev_max == host_max, kind
+        n_blocks = -(-c["encoded_exponent"].size // 4096)
+        used = 64 + 2048 * 8 + 2048 + 4 * (8 * n_blocks + 1)      # the rest is alignment padding
+        assert np.array_equal(dev.cpu().numpy()[:used], host[:used]), kind
 
 
 @pytest.mark.parametrize("pad", [1, 2, 4, 7])
@@ -133,17 +143,18 @@ def test_gpu_side_stream_and_repeat():
     w2 = make_case("laplace", 300_000, 101)
     c1, c2 = compress_product(w1), compress_product(w2)
     g1, g2 = to_gpu(c1), to_gpu(c2)
-    t1, t2 = D.build_tables(g1["luts"]), D.build_tables(g2["luts"])
+    (t1, m1), (t2, m2) = (D.prepare(g["luts"], g["encoded_exponent"], g["output_positions"], g["gaps"], w.size)
+                          for g, w in ((g1, w1), (g2, w2)))
     out = torch.empty(max(w1.size, w2.size), dtype=torch.bfloat16, device=DEV)
     torch.cuda.synchronize()
     s = torch.cuda.Stream()
     with torch.cuda.stream(s):
         for _ in range(3):   # same output buffer reused, stream order is the only guard
             D.decode(g1["luts"], g1["encoded_exponent"], g1["sign_mantissa"], g1["output_positions"],
-                     g1["gaps"], out, t1, max_elems_per_block(c1["output_positions"]))
+                     g1["gaps"], out, t1, m1)
             a = out[: w1.size].clone()
             D.decode(g2["luts"], g2["encoded_exponent"], g2["sign_mantissa"], g2["output_positions"],
-                     g2["gaps"], out, t2, max_elems_per_block(c2["output_positions"]))
+                     g2["gaps"], out, t2, m2)
             b = out[: w2.size].clone()
     s.synchronize()
     assert np.array_equal(a.view(torch.int16).cpu().numpy().view(np.uint16), w1)
@@ -175,9 +186,9 @@ def test_gpu_llama_block_round_trip():
     wu = w.view(torch.int16).cpu().numpy().view(np.uint16)
     c = compress_product(wu)
     g = to_gpu(c)
-    tables = D.build_tables(g["luts"])
+    ws, max_sub = D.prepare(g["luts"], g["encoded_exponent"], g["output_positions"], g["gaps"], w.numel())
     out = torch.empty_like(w)
     D.decode(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
-             out, tables, max_elems_per_block(c["output_positions"]))
+             out, ws, max_sub)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), w.view(torch.int16))
