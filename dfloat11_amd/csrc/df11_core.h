@@ -341,8 +341,9 @@ DF11_HD uint32_t thread_quota(uint32_t excl, uint32_t count, uint32_t n_out) {
 // Four BF16 words from four exponent bytes E and four sign|mantissa bytes S:
 // high bytes (S & 0x80) | (E >> 1), low bytes (E << 7) | (S & 0x7f), interleaved.
 DF11_HD void merge4(uint32_t E, uint32_t S, uint32_t& out01, uint32_t& out23) {
-  const uint32_t hi = (S & 0x80808080u) | ((E >> 1) & 0x7f7f7f7fu);
-  const uint32_t lo = ((E << 7) & 0x80808080u) | (S & 0x7f7f7f7fu);
+  constexpr uint32_t kTop = 0x80808080u;   // bit 7 of every byte
+  const uint32_t hi = (S & kTop) | ((E >> 1) & ~kTop);
+  const uint32_t lo = ((E << 7) & kTop) | (S & ~kTop);
 #if defined(__HIP_DEVICE_COMPILE__)
   out01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);   // lo0 hi0 lo1 hi1
   out23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);   // lo2 hi2 lo3 hi3
@@ -376,15 +377,19 @@ DF11_HD SubSpans spans_of(const SubPlan& p) {
   return s;
 }
 
+// Eight BF16 words from 8 staging bytes `e` and 8 sign|mantissa bytes `m`.
+DF11_HD U32x4 merge8(const U32x2& e, const U32x2& m) {
+  U32x4 o;
+  merge4(e.x, m.x, o.x, o.y);
+  merge4(e.y, m.y, o.z, o.w);
+  return o;
+}
+
 // Body group g: 8 staging bytes + 8 sign|mantissa bytes `m` -> 16 bytes of BF16.
 DF11_HD void stream_group(uint32_t g, const SubPlan& p, const uint8_t* stage, const U32x2& m,
                           uint16_t* out) {
   const uint32_t s0 = g * (uint32_t)kGroup;
-  const U32x2 e = load_as<U32x2>(stage + s0);
-  U32x4 o;
-  merge4(e.x, m.x, o.x, o.y);
-  merge4(e.y, m.y, o.z, o.w);
-  store_as<U32x4>(out + p.a0 + s0, o);
+  store_as<U32x4>(out + p.a0 + s0, merge8(load_as<U32x2>(stage + s0), m));
 }
 
 // One element of a head or tail (or of everything, for unaligned buffers).

@@ -153,14 +153,49 @@ __global__ __launch_bounds__(kThreads) void index_kernel(const IndexArgs a) {
 // ---------------------------------------------------------------------------
 // Decode kernel.
 // LDS layout (dynamic): tables | byte LUT rows + length row | 8 staging areas
+//
+// Everything that is the same for the 64 lanes of a wavefront (sub-block index,
+// output position, plan of the write-out) is kept wavefront-uniform on purpose,
+// so that it lives in scalar registers and costs no vector instructions; global
+// addresses are a uniform 64-bit base plus a 32-bit lane offset.
 // ---------------------------------------------------------------------------
-struct DecodeArgs {
-  const uint8_t* luts;
-  const uint8_t* codes;
-  const uint8_t* sign_mantissa;
-  const uint8_t* gaps;
-  uint16_t* out;
-  const uint8_t* ws;
+// A zero the compiler cannot see through, held in a vector register: adding it to
+// a uniform index keeps the access a vector load.
+__device__ __forceinline__ uint32_t opaque_vector_zero() {
+  uint32_t z;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+  return z;
+}
+
+// Two consecutive 32-bit words at a 4-byte aligned address.
+__device__ __forceinline__ U32x2 load_as_unaligned_pair(const uint32_t* p) {
+  U32x2 v;
+  v.x = p[0];
+  v.y = p[1];
+  return v;
+}
+
+// Marks loaded values as used at this point of the program, so that the wait for
+// their arrival is placed here and not at their first real use.
+__device__ __forceinline__ void claim(uint32_t& v) { asm volatile("" : "+v"(v)); }
+template <class... T>
+__device__ __forceinline__ void claim(uint32_t& v, T&... rest) {
+  claim(v);
+  claim(rest...);
+}
+
+// 16-byte store of output that is written once and not read again by this kernel.
+typedef uint32_t V4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_stream(uint16_t* p, const U32x4& v) {
+#if defined(DF11_NT_STORES)
+  const V4u x = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(x, reinterpret_cast<V4u*>(p));
+#else
+  store_as<U32x4>(p, v);
+#endif
+}
+
+struct DecodeSizes {
   int64_t n_bytes;
   int64_t n_elements;
   int64_t n_blocks;
@@ -173,79 +208,138 @@ struct DecodeArgs {
 
 constexpr int kPrefetchGroups = 3;   // body groups per lane whose sign|mantissa bytes are requested early
 
+__device__ __forceinline__ uint32_t uniform(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
+}
+
+// Inputs of one sub-block exactly as loaded: nothing here is computed on, so
+// requesting them one sub-block ahead never waits for them.
 struct SubInputs {
-  Chunk c;
-  uint32_t gap;
-  uint32_t base;       // first output element
-  uint32_t end_hint;   // first output element of the next sub-block
+  uint32_t d0, d1, d2;   // bytes [0,4), [4,8), [8,12) of the lane's chunk, little-endian words
+  uint32_t gap_raw;      // two bytes of the packed gaps, little-endian
+  uint32_t base;         // first output element (same in every lane)
+  uint32_t end_hint;     // first output element of the next sub-block (same in every lane)
 };
 
-__device__ __forceinline__ SubInputs fetch_sub(const DecodeArgs& a, const uint32_t* subpos, int64_t sub,
-                                               int lane, int64_t n_gap_bytes) {
+// Bytes [8*lane, 8*lane + 12) of sub-block `sub` (uniform), its two gap bytes and
+// its output position.  gap_byte: lane's byte offset inside the sub-block's 40
+// bytes of gaps, chosen so that byte + 1 stays inside them.
+__device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes,
+                                               const uint8_t* __restrict__ gaps,
+                                               const uint32_t* __restrict__ subpos,
+                                               const DecodeSizes& z, int64_t sub, uint32_t lane,
+                                               uint32_t gap_byte, uint32_t vector_zero) {
   SubInputs in;
-  const int64_t gid = sub * kLanes + lane;
-  in.c = fetch_chunk(a.codes, a.n_bytes, gid, a.codes_aligned != 0);
-  in.gap = gap_of(a.gaps, gid, n_gap_bytes);
-  in.base = subpos[sub];
-  in.end_hint = subpos[sub + 1];
+  const int64_t sub_off = sub * kSubBytes;                       // uniform
+  if (z.codes_aligned && sub_off + kSubBytes + 4 <= z.n_bytes) {   // uniform: whole sub-block + look-ahead in range
+    const uint8_t* p = codes + sub_off + lane * (uint32_t)kChunkBytes;
+    const U32x2 v = load_as<U32x2>(p);
+    in.d0 = v.x;
+    in.d1 = v.y;
+    in.d2 = load_as<uint32_t>(p + 8);
+  } else {
+    const Chunk c = fetch_chunk(codes, z.n_bytes, sub * kLanes + lane, false);
+    in.d0 = __builtin_bswap32(c.hi);
+    in.d1 = __builtin_bswap32(c.lo);
+    in.d2 = __builtin_bswap32(c.next);
+  }
+  uint16_t g16;
+  __builtin_memcpy(&g16, gaps + sub * (kLanes * 5 / 8) + gap_byte, 2);   // unaligned 2-byte load
+  in.gap_raw = g16;
+  // Loaded per lane although the index is uniform: a scalar load would share its
+  // wait counter with the LDS lookups and stall the first of them.  The value is
+  // made uniform where it is consumed, not here: that would wait for the load one
+  // sub-block too early.
+  const U32x2 pos = load_as_unaligned_pair(subpos + sub + vector_zero);
+  in.base = pos.x;
+  in.end_hint = pos.y;
   return in;
 }
 
-__global__ __launch_bounds__(kThreads) void decode_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(kThreads) void decode_kernel(
+    const uint8_t* __restrict__ luts, const uint8_t* __restrict__ codes,
+    const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
+    uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
   extern __shared__ __align__(16) uint8_t lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_rows = min(a.n_luts - 1, kMaxDecodeRows);
+  const int tid = threadIdx.x;
+  const uint32_t lane = tid & 63;
+  const uint32_t wave = uniform(tid >> 6);
+  const int n_rows = min(z.n_luts - 1, kMaxDecodeRows);
   uint8_t* lds_tables = lds;
   uint8_t* lds_rows = lds + kTablesBytes;
-  uint8_t* stage = lds_rows + (kMaxDecodeRows + 1) * 256 + (size_t)wave * a.stage_cap;
+  uint8_t* stage = lds_rows + (kMaxDecodeRows + 1) * 256 + wave * (uint32_t)z.stage_cap;
   {
-    const uint4* src = reinterpret_cast<const uint4*>(a.ws + kWsTablesOffset);
+    const uint4* src = reinterpret_cast<const uint4*>(ws + kWsTablesOffset);
     uint4* dst = reinterpret_cast<uint4*>(lds_tables);
     for (int i = tid; i < kTablesBytes / 16; i += kThreads) dst[i] = src[i];
-    stage_rows(a.luts, a.n_luts, n_rows, lds_rows, tid, kThreads);
+    stage_rows(luts, z.n_luts, n_rows, lds_rows, tid, kThreads);
   }
   __syncthreads();   // the only workgroup barrier: tables are read-only from here on
 
   const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
   const Luts l{lds_rows, n_rows};
-  const int64_t n_gap_bytes = a.n_blocks * kGapBytesPerBlock;
-  const uint32_t* subpos = reinterpret_cast<const uint32_t*>(a.ws + kWsSubposOffset);
-  const bool vec_ok = a.vec_ok != 0;
+  const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
+  const bool vec_ok = z.vec_ok != 0;
   const int64_t stride = (int64_t)gridDim.x * kWavesPerGroup;
 
-  int64_t sub = (int64_t)blockIdx.x * kWavesPerGroup + wave;
-  if (sub >= a.n_subs) return;
-  SubInputs cur = fetch_sub(a, subpos, sub, lane, n_gap_bytes);
+  // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
+  // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
+  // its window starts one byte early and never reaches past them.
+  const uint32_t gap_bit = lane * 5u;
+  const uint32_t gap_byte = min(gap_bit >> 3, (uint32_t)(kLanes * 5 / 8 - 2));
+  const uint32_t gap_shift = 11u - (gap_bit - 8u * gap_byte);
 
-  for (; sub < a.n_subs; sub += stride) {
+  int64_t sub = (int64_t)blockIdx.x * kWavesPerGroup + wave;   // uniform
+  if (sub >= z.n_subs) return;
+  const uint32_t vzero = opaque_vector_zero();
+  SubInputs cur = fetch_sub(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
+  claim(cur.d0, cur.d1, cur.d2, cur.gap_raw, cur.base, cur.end_hint);   // see the claim inside the loop
+
+  for (; sub < z.n_subs; sub += stride) {
     // ---- requests whose latency the two decode passes hide: the next
     // sub-block's inputs and this one's sign|mantissa bytes
     const int64_t next_sub = sub + stride;
     SubInputs nxt = cur;
-    if (next_sub < a.n_subs) nxt = fetch_sub(a, subpos, next_sub, lane, n_gap_bytes);
+    if (next_sub < z.n_subs) nxt = fetch_sub(codes, gaps, subpos, z, next_sub, lane, gap_byte, vzero);
 
-    const int64_t base = cur.base;
-    const int64_t a0 = base & ~(int64_t)(kGroup - 1);
-    int64_t end_hint = cur.end_hint;
-    if (end_hint > a.n_elements) end_hint = a.n_elements;
-    const uint32_t first_body = (base != a0) ? 1u : 0u;   // group 0 is a partial head unless aligned
+    const uint32_t base = uniform(cur.base);
+    const uint32_t a0 = base & ~(uint32_t)(kGroup - 1);
+    const uint32_t n_total = (uint32_t)z.n_elements;          // < 2^32, checked by the host
+    const uint32_t end_hint = min(uniform(cur.end_hint), n_total);
+    const uint32_t hint_len = end_hint > a0 ? end_hint - a0 : 0u;   // staging index one past the hinted end
+    const uint32_t first_body = (base != a0) ? 1u : 0u;       // group 0 is a partial head unless aligned
+    const uint8_t* sm0 = sign_mantissa + a0;                  // uniform bases
+    uint16_t* out0 = out + a0;
     U32x2 m[kPrefetchGroups];
 #pragma unroll
     for (int k = 0; k < kPrefetchGroups; ++k) {
       m[k] = U32x2{0, 0};
-      const int64_t e0 = a0 + (int64_t)(first_body + lane + kLanes * k) * kGroup;
-      if (vec_ok && e0 + kGroup <= end_hint) m[k] = load_as<U32x2>(a.sign_mantissa + e0);
+      const uint32_t s0 = (first_body + lane + (uint32_t)(kLanes * k)) * (uint32_t)kGroup;
+      if (vec_ok && s0 + (uint32_t)kGroup <= hint_len) m[k] = load_as<U32x2>(sm0 + s0);
     }
+    // The ragged ends, fewer than 8 elements each: lanes 0..7 take the head, lanes
+    // 8..15 the tail, one element per lane, its sign|mantissa byte requested now.
+    const uint32_t phase0 = base - a0;
+    const uint32_t head_end_hint = phase0 ? min((uint32_t)kGroup, hint_len) : 0u;
+    const uint32_t tail_begin_hint = max(hint_len & ~(uint32_t)(kGroup - 1), head_end_hint);
+    const uint32_t edge_hint = lane < (uint32_t)kGroup ? phase0 + lane : tail_begin_hint + lane - (uint32_t)kGroup;
+    const bool edge_hint_ok = vec_ok && lane < 2u * kGroup &&
+                              (lane < (uint32_t)kGroup ? edge_hint < head_end_hint : edge_hint < hint_len);
+    uint32_t edge_byte = 0;
+    if (edge_hint_ok) edge_byte = sm0[edge_hint];
 
     // ---- pass 1 and the exclusive offsets inside the wavefront
-    const uint32_t count = count_chunk(t, l, cur.c.hi, cur.c.lo, cur.c.next, cur.gap);
+    const Chunk c{__builtin_bswap32(cur.d0), __builtin_bswap32(cur.d1), __builtin_bswap32(cur.d2)};
+    const uint32_t gap_word = __builtin_bswap32(cur.gap_raw) >> 16;   // the two bytes, big-endian
+    const uint32_t gap = (gap_word >> gap_shift) & 31u;
+    const uint32_t count = count_chunk(t, l, c.hi, c.lo, c.next, gap);
     const uint32_t incl = wave_inclusive_scan(count);
-    const uint32_t total = wave_total(incl);
+    const uint32_t total = wave_total(incl);                  // uniform
     const uint32_t excl = incl - count;
 
     // ---- pass 2: decode into this wavefront's staging area, in output order
-    const SubPlan p = plan_sub(base, total, a.n_elements, a.stage_cap);
-    emit_chunk(t, l, cur.c.hi, cur.c.lo, cur.c.next, cur.gap, thread_quota(excl, count, p.n_out),
+    const SubPlan p = plan_sub((int64_t)base, total, z.n_elements, z.stage_cap);   // uniform
+    emit_chunk(t, l, c.hi, c.lo, c.next, gap, thread_quota(excl, count, p.n_out),
                stage + p.phase + excl);
     // Staging is exchanged between the lanes of one wavefront only; its LDS
     // operations execute in order, the fence keeps the compiler from reordering.
@@ -254,29 +348,54 @@ __global__ __launch_bounds__(kThreads) void decode_kernel(const DecodeArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     // ---- stream out
-    const SubSpans sp = spans_of(p);
-    if (vec_ok) {
-      for (uint32_t i = sp.head_begin + lane; i < sp.head_end; i += kLanes)
-        stream_element(i, p, stage, a.sign_mantissa, a.out);
+    // Vector loads and stores share one in-order completion counter on this
+    // hardware, so the first use of a loaded value after a store waits for that
+    // store to reach memory.  Every value requested above is therefore claimed
+    // here, before the first store of this sub-block is issued; by now those
+    // loads are a whole decode old and the wait costs nothing.
+    claim(nxt.d0, nxt.d1, nxt.d2, nxt.gap_raw, nxt.base, nxt.end_hint);
+#pragma unroll
+    for (int k = 0; k < kPrefetchGroups; ++k) claim(m[k].x, m[k].y);
+    claim(edge_byte);
+
+    const SubSpans sp = spans_of(p);                          // uniform
+    if (vec_ok && p.phase + p.n_out == hint_len) {
+      // The hint was exact (it always is for a well-formed workspace): every
+      // sign|mantissa byte of the first 3 x 64 groups and of the ragged ends is in
+      // registers, and the stores below are not interleaved with loads.
+      U32x4 o[kPrefetchGroups];
       uint32_t g = sp.body_begin + lane;
 #pragma unroll
-      for (int k = 0; k < kPrefetchGroups; ++k, g += kLanes) {
-        if (g < sp.body_end) {
-          // requested early only when the hint covered the group; the hint is the
-          // next sub-block's start, which equals this one's end for a valid stream
-          const int64_t e0 = p.a0 + (int64_t)g * kGroup;
-          const bool early = sp.body_begin == first_body && e0 + kGroup <= end_hint;
-          const U32x2 mm = early ? m[k] : load_as<U32x2>(a.sign_mantissa + e0);
-          stream_group(g, p, stage, mm, a.out);
-        }
+      for (int k = 0; k < kPrefetchGroups; ++k) {
+        const uint32_t gk = g + (uint32_t)(kLanes * k);
+        const uint32_t s0 = (gk < sp.body_end ? gk : 0u) * (uint32_t)kGroup;   // in range for idle lanes too
+        o[k] = merge8(load_as<U32x2>(stage + s0), m[k]);
       }
-      for (; g < sp.body_end; g += kLanes)
-        stream_group(g, p, stage, load_as<U32x2>(a.sign_mantissa + p.a0 + (int64_t)g * kGroup), a.out);
-      for (uint32_t i = sp.tail_begin + lane; i < sp.tail_end; i += kLanes)
-        stream_element(i, p, stage, a.sign_mantissa, a.out);
+      const bool is_head = lane < (uint32_t)kGroup;
+      const uint32_t edge = is_head ? sp.head_begin + lane : sp.tail_begin + lane - (uint32_t)kGroup;
+      const bool edge_on = lane < 2u * kGroup && edge < (is_head ? sp.head_end : sp.tail_end);
+      const uint16_t edge_word = merge(stage[edge_on ? edge : 0u], edge_byte);
+#pragma unroll
+      for (int k = 0; k < kPrefetchGroups; ++k) {
+        const uint32_t gk = g + (uint32_t)(kLanes * k);
+        if (gk < sp.body_end) store_stream(out0 + gk * (uint32_t)kGroup, o[k]);
+      }
+      if (edge_on) out0[edge] = edge_word;
+      // sub-blocks of more than 3 x 64 groups (long runs of very short codes)
+      for (g += (uint32_t)(kLanes * kPrefetchGroups); g < sp.body_end; g += kLanes) {
+        const uint32_t s0 = g * (uint32_t)kGroup;
+        store_stream(out0 + s0, merge8(load_as<U32x2>(stage + s0), load_as<U32x2>(sm0 + s0)));
+      }
+    } else if (vec_ok) {
+      for (uint32_t i = sp.head_begin + lane; i < sp.head_end; i += kLanes) out0[i] = merge(stage[i], sm0[i]);
+      for (uint32_t g = sp.body_begin + lane; g < sp.body_end; g += kLanes) {
+        const uint32_t s0 = g * (uint32_t)kGroup;
+        store_stream(out0 + s0, merge8(load_as<U32x2>(stage + s0), load_as<U32x2>(sm0 + s0)));
+      }
+      for (uint32_t i = sp.tail_begin + lane; i < sp.tail_end; i += kLanes) out0[i] = merge(stage[i], sm0[i]);
     } else {
       for (uint32_t i = p.phase + lane; i < p.phase + p.n_out; i += kLanes)
-        stream_element(i, p, stage, a.sign_mantissa, a.out);
+        out0[i] = merge(stage[i], sm0[i]);
     }
     // The next sub-block's staging stores must not pass this one's loads.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -430,30 +549,26 @@ int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint
   DeviceInfo info;
   if (int rc = device_info(info)) return rc;
 
-  DecodeArgs a;
-  a.luts = luts;
-  a.codes = encoded_exponent;
-  a.sign_mantissa = sign_mantissa;
-  a.gaps = gaps;
-  a.out = outputs;
-  a.ws = static_cast<const uint8_t*>(workspace);
-  a.n_bytes = n_bytes;
-  a.n_elements = n_elements;
-  a.n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
-  a.n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
-  a.n_luts = n_luts;
-  a.stage_cap = ((max_elems_per_subblock + kGroup + 15) / 16) * 16;   // + up to 7 elements of output phase
-  a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
-  a.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
+  if (n_elements >= ((int64_t)1 << 32)) return DF11_ERR_UNSUPPORTED;   // positions are u32
+  DecodeSizes z;
+  z.n_bytes = n_bytes;
+  z.n_elements = n_elements;
+  z.n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  z.n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
+  z.n_luts = n_luts;
+  z.stage_cap = ((max_elems_per_subblock + kGroup + 15) / 16) * 16;   // + up to 7 elements of output phase
+  z.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
+  z.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
              (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
 
-  const size_t lds_bytes = (size_t)kFixedLds + (size_t)kWavesPerGroup * (size_t)a.stage_cap;
+  const size_t lds_bytes = (size_t)kFixedLds + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
-  const int64_t needed = (a.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
+  const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
 
   hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes,
-                     static_cast<hipStream_t>(stream), a);
+                     static_cast<hipStream_t>(stream), luts, encoded_exponent, sign_mantissa, gaps,
+                     outputs, static_cast<const uint8_t*>(workspace), z);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? DF11_OK : hip_fail(e);
 }
