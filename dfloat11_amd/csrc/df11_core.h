@@ -243,6 +243,106 @@ DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo
   }
 }
 
+// ---- one decode per chunk, kept in registers -------------------------------------
+// The fast path decodes a chunk once.  The lookups of a chunk are few (each
+// resolves up to four codes), so their results fit in registers: kMainSlots
+// lookups that stay inside the chunk plus kTailSlots for the codes that reach
+// into the look-ahead.  Once the lane's output offset is known, the symbols are
+// replayed into the staging area with no further table access.  A chunk that
+// needs more lookups than there are slots reports `overflow` and is handled by
+// count_chunk / emit_chunk instead.
+constexpr int kMainSlots = 8;
+constexpr int kTailSlots = 3;
+constexpr int kSlots = kMainSlots + kTailSlots;
+
+struct ChunkSyms {
+  uint32_t syms[kSlots];   // symbol bytes of lookup i, first code in byte 0, unused bytes zero
+  uint32_t ks;             // 3 bits per lookup: how many symbols it contributes (0..4)
+  uint32_t count;          // codes that start in the chunk
+  bool overflow;           // ran out of slots: count and syms are incomplete
+};
+
+DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo,
+                                    uint32_t next, uint32_t gap) {
+  ChunkSyms r;
+  uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
+  uint32_t c = gap, n = 0, ks = 0;
+#pragma unroll
+  for (int i = 0; i < kMainSlots; ++i) {
+    r.syms[i] = 0;
+    if (c <= 64u - (uint32_t)kK) {          // the lookup stays inside the chunk
+      const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+      uint32_t syms = e.x, meta = e.y;
+      if (meta == 0u) {
+        uint32_t len;
+        walk(l, with_next(w, next, c), syms, len);
+        meta = len | 0x100u;
+        DF11_KEEP_BRANCH();
+      }
+      r.syms[i] = syms;
+      const uint32_t k = meta >> 8;
+      ks |= k << (3 * i);
+      n += k;
+      w <<= (meta & 63u);
+      c += meta & 0xffu;
+    }
+  }
+  r.overflow = c <= 64u - (uint32_t)kK;
+  uint32_t todo = 0;                          // codes that still start before the chunk ends
+  if (!r.overflow && c < 64u) {
+    todo = t.cntt[(1u << (64u - c)) | (uint32_t)(w >> c)];
+    w = with_next(w, next, c);
+  }
+#pragma unroll
+  for (int i = 0; i < kTailSlots; ++i) {
+    r.syms[kMainSlots + i] = 0;
+    if (todo) {
+      const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+      uint32_t syms = e.x, meta = e.y;
+      if (meta == 0u) {
+        uint32_t len;
+        walk(l, w, syms, len);
+        meta = len | 0x100u;
+      }
+      r.syms[kMainSlots + i] = syms;
+      const uint32_t k = meta >> 8;
+      const uint32_t take = k < todo ? k : todo;
+      ks |= take << (3 * (kMainSlots + i));
+      n += take;
+      todo -= take;
+      w <<= (meta & 63u);
+    }
+  }
+  r.overflow = r.overflow || todo != 0u;
+  r.ks = ks;
+  r.count = n;
+  return r;
+}
+
+// Write the chunk's r.count symbols to p[0..count).  While four or more bytes
+// remain, a lookup stores its four bytes at once (the bytes past its symbols are
+// zero and are overwritten by the next store); the last one to three symbols are
+// gathered and stored exactly, so nothing is written at or beyond p + count.
+DF11_HD void replay_chunk(const ChunkSyms& r, uint8_t* p) {
+  uint32_t rem = r.count, acc = 0, got = 0;
+#pragma unroll
+  for (int i = 0; i < kSlots; ++i) {
+    const uint32_t k = (r.ks >> (3 * i)) & 7u;
+    if (rem >= 4u) {
+      store32(p, r.syms[i]);
+      p += k;
+      rem -= k;
+    } else {
+      acc |= r.syms[i] << got;
+      got += 8u * k;
+    }
+  }
+  if (rem < 4u) {                 // rem == 4 can only be left by a chunk that overflowed its slots
+    if (rem & 2u) store16(p, acc);
+    if (rem & 1u) p[rem & 2u] = (uint8_t)(acc >> (8u * (rem & 2u)));
+  }
+}
+
 // BF16 word from exponent byte and sign|mantissa byte.
 DF11_HD uint16_t merge(uint32_t exponent, uint32_t sm) {
   return (uint16_t)(((sm & 0x80u) << 8) | (exponent << 7) | (sm & 0x7fu));

@@ -9,10 +9,13 @@
 // (tables are copied into LDS once per workgroup).  Per sub-block a wavefront
 //   1. takes its chunk (+4 bytes of look-ahead), gap and start index, all fetched
 //      one sub-block ahead, and requests the sign|mantissa bytes it will need;
-//   2. counts the codes starting in each lane's chunk (four-symbol table in LDS);
+//   2. decodes each lane's chunk once (four-symbol table in LDS); the handful of
+//      lookups a chunk needs stay in registers, and their count is the lane's
+//      number of codes;
 //   3. turns the 64 counts into exclusive offsets with a DPP scan;
-//   4. decodes again, storing the symbols of each lookup with one unaligned
-//      32-bit store into its private LDS staging area, in output order;
+//   4. replays the lookups from registers into its private LDS staging area, in
+//      output order (chunks with too many lookups for the registers fall back to
+//      counting first and decoding a second time);
 //   5. streams the staging area out: 8 exponent bytes (LDS) + 8 sign|mantissa
 //      bytes -> one 16-byte BF16 store per lane, contiguous across the wavefront.
 #include <hip/hip_runtime.h>
@@ -51,6 +54,10 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
   v = dpp_add<0x142, 0xa, 0xf, false>(v);   // row_bcast:15 into rows 1 and 3
   v = dpp_add<0x143, 0xc, 0xf, false>(v);   // row_bcast:31 into rows 2 and 3
   return v;
+}
+
+__device__ __forceinline__ bool wave_all(bool pred) {
+  return __builtin_amdgcn_ballot_w64(pred) == __builtin_amdgcn_ballot_w64(true);
 }
 
 __device__ __forceinline__ uint32_t wave_total(uint32_t inclusive) {
@@ -328,19 +335,27 @@ __global__ __launch_bounds__(kThreads) void decode_kernel(
     uint32_t edge_byte = 0;
     if (edge_hint_ok) edge_byte = sm0[edge_hint];
 
-    // ---- pass 1 and the exclusive offsets inside the wavefront
+    // ---- decode, and the exclusive offsets inside the wavefront
     const Chunk c{__builtin_bswap32(cur.d0), __builtin_bswap32(cur.d1), __builtin_bswap32(cur.d2)};
     const uint32_t gap_word = __builtin_bswap32(cur.gap_raw) >> 16;   // the two bytes, big-endian
     const uint32_t gap = (gap_word >> gap_shift) & 31u;
-    const uint32_t count = count_chunk(t, l, c.hi, c.lo, c.next, gap);
+    // One decode per chunk, results held in registers.  If any lane of the
+    // wavefront ran out of register slots, or may not write all its symbols (end
+    // of the tensor), the wavefront takes the two-pass route instead.
+    const ChunkSyms cs = decode_chunk_regs(t, l, c.hi, c.lo, c.next, gap);
+    const bool all_fit = wave_all(!cs.overflow);
+    const uint32_t count = all_fit ? cs.count : count_chunk(t, l, c.hi, c.lo, c.next, gap);
     const uint32_t incl = wave_inclusive_scan(count);
     const uint32_t total = wave_total(incl);                  // uniform
     const uint32_t excl = incl - count;
 
-    // ---- pass 2: decode into this wavefront's staging area, in output order
+    // ---- symbols to their place in the staging area, in output order
     const SubPlan p = plan_sub((int64_t)base, total, z.n_elements, z.stage_cap);   // uniform
-    emit_chunk(t, l, c.hi, c.lo, c.next, gap, thread_quota(excl, count, p.n_out),
-               stage + p.phase + excl);
+    const uint32_t quota = thread_quota(excl, count, p.n_out);
+    if (all_fit && wave_all(quota == count))
+      replay_chunk(cs, stage + p.phase + excl);
+    else
+      emit_chunk(t, l, c.hi, c.lo, c.next, gap, quota, stage + p.phase + excl);
     // Staging is exchanged between the lanes of one wavefront only; its LDS
     // operations execute in order, the fence keeps the compiler from reordering.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

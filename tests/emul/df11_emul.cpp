@@ -90,7 +90,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
                                 const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
                                 int n_luts, int64_t n_bytes, int64_t n_elements,
                                 int max_elems_per_sub, int grid, int codes_misalign,
-                                int out_misalign) {
+                                int out_misalign, int flags) {
   if (max_elems_per_sub <= 0 || max_elems_per_sub > kMaxElemsPerSub) max_elems_per_sub = kMaxElemsPerSub;
   const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
   const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
@@ -129,29 +129,46 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
 
   std::vector<Chunk> chunk(kLanes);
   std::vector<uint32_t> gap(kLanes), count(kLanes), excl(kLanes);
+  std::vector<ChunkSyms> regs(kLanes);
+  const bool force_two_pass = (flags & 1) != 0;   // exercise the fall-back route on any input
+  const bool force_check = true;
   for (int64_t wave_gid = 0; wave_gid < stride; ++wave_gid) {
     for (int64_t sub = wave_gid; sub < n_subs; sub += stride) {
-      uint32_t total = 0;
+      // one decode per chunk into "registers"; the wavefront falls back to the
+      // two-pass route if any lane overflowed its slots or may not write everything
+      bool all_fit = true;
       for (int lane = 0; lane < kLanes; ++lane) {
         const int64_t gid = sub * kLanes + lane;
         chunk[lane] = fetch_chunk(codes_p, n_bytes, gid, codes_aligned);
         gap[lane] = gap_of(c_gaps.p, gid, n_gap_bytes);
-        count[lane] = count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
+        regs[lane] = decode_chunk_regs(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
+        all_fit = all_fit && !regs[lane].overflow;
+      }
+      uint32_t total = 0;
+      for (int lane = 0; lane < kLanes; ++lane) {
+        count[lane] = all_fit ? regs[lane].count
+                              : count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
+        if (all_fit && force_check)   // the two routes must agree on the count
+          if (count[lane] != count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane])) return 7;
         excl[lane] = total;
         total += count[lane];
       }
       const SubPlan p = plan_sub((int64_t)subpos[sub], total, n_elements, stage_cap);
+      bool replay = all_fit && !force_two_pass;
+      for (int lane = 0; lane < kLanes; ++lane)
+        replay = replay && thread_quota(excl[lane], count[lane], p.n_out) == count[lane];
       memset(stage.p, 0xDD, (size_t)stage_cap);
       // Lanes run concurrently on the device, so no lane may rely on a later lane
-      // repairing what it wrote.  Even sub-blocks emit in ascending lane order,
+      // repairing what it wrote.  Even sub-blocks write in ascending lane order,
       // odd ones in descending order: a store that strays into a neighbour's
       // bytes corrupts the result in one of the two.
       for (int k = 0; k < kLanes; ++k) {
         const int lane = (sub & 1) ? kLanes - 1 - k : k;
         const uint32_t quota = thread_quota(excl[lane], count[lane], p.n_out);
         // a lane with nothing to write may hold an out-of-range pointer; it must not use it
-        emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota,
-                   quota ? stage.p + p.phase + excl[lane] : nullptr);
+        uint8_t* dst = quota ? stage.p + p.phase + excl[lane] : nullptr;
+        if (replay) replay_chunk(regs[lane], dst);
+        else emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota, dst);
       }
       const SubSpans sp = spans_of(p);
       if (vec_ok) {
@@ -170,7 +187,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
 
 #ifdef DF11_EMUL_MAIN
 // Stand-alone driver (built with AddressSanitizer): reads one case from a file
-//   i64 n_luts, n_bytes, n_elements, n_blocks, max_elems, grid, codes_misalign, out_misalign
+//   i64 n_luts, n_bytes, n_elements, n_blocks, max_elems, grid, codes_misalign, out_misalign, flags
 //   luts | codes | sign_mantissa | positions (n_blocks u32) | gaps
 // and writes the decoded u16 words to the output file.
 #include <cstdio>
@@ -178,8 +195,8 @@ int main(int argc, char** argv) {
   if (argc != 3) return 2;
   FILE* f = fopen(argv[1], "rb");
   if (!f) return 2;
-  int64_t h[8];
-  if (fread(h, 8, 8, f) != 8) return 2;
+  int64_t h[9];
+  if (fread(h, 8, 9, f) != 9) return 2;
   const int64_t n_luts = h[0], n_bytes = h[1], n_elements = h[2], n_blocks = h[3];
   Exact<uint8_t> luts((size_t)n_luts * 256), codes((size_t)n_bytes), sm((size_t)n_elements);
   Exact<uint32_t> pos((size_t)n_blocks);
@@ -193,7 +210,7 @@ int main(int argc, char** argv) {
   fclose(f);
   if (!ok) return 2;
   int rc = df11_emul_decode(luts.p, codes.p, sm.p, pos.p, gaps.p, out.p, (int)n_luts, n_bytes,
-                            n_elements, (int)h[4], (int)h[5], (int)h[6], (int)h[7]);
+                            n_elements, (int)h[4], (int)h[5], (int)h[6], (int)h[7], (int)h[8]);
   if (rc) return 3;
   FILE* g = fopen(argv[2], "wb");
   if (!g) return 2;

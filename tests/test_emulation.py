@@ -19,7 +19,7 @@ def emul():
     subprocess.run(["make", "-s", "-C", EMUL_DIR], check=True)
     L = ctypes.CDLL(os.path.join(EMUL_DIR, "libdf11_emul.so"))
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
-    L.df11_emul_decode.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, i32, i32]
+    L.df11_emul_decode.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, i32, i32, i32]
     L.df11_emul_decode.restype = i32
     return L
 
@@ -28,18 +28,19 @@ def _p(a):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0):
+def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0, two_pass=False):
     n = c["sign_mantissa"].size
     out = np.zeros(n, np.uint16)
     luts = np.ascontiguousarray(c["luts"])
     rc = L.df11_emul_decode(_p(luts), _p(c["encoded_exponent"]), _p(c["sign_mantissa"]),
                             _p(c["output_positions"]), _p(c["gaps"]), _p(out), luts.shape[0],
-                            c["encoded_exponent"].size, n, max_elems, grid, codes_misalign, out_misalign)
+                            c["encoded_exponent"].size, n, max_elems, grid, codes_misalign, out_misalign,
+                            1 if two_pass else 0)
     assert rc == 0
     return out
 
 
-def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=None):
+def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=None, two_pass=False):
     n = c["sign_mantissa"].size
     n_bytes = c["encoded_exponent"].size
     n_blocks = -(-n_bytes // 4096)
@@ -47,7 +48,7 @@ def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=
     inp, outp = str(tmp_path / "case.bin"), str(tmp_path / "out.bin")
     with open(inp, "wb") as f:
         f.write(np.array([luts.shape[0], n_bytes, n, n_blocks, max_elems, grid, codes_misalign,
-                          out_misalign], np.int64).tobytes())
+                          out_misalign, 1 if two_pass else 0], np.int64).tobytes())
         f.write(luts.tobytes())
         f.write(c["encoded_exponent"].tobytes())
         f.write(c["sign_mantissa"].tobytes())
@@ -69,8 +70,8 @@ def test_emulated_kernel_matches_oracle(emul, oracle, kind, n):
     assert np.array_equal(ref, w)
     got = run_emul(emul, c, max_elems=max_elems_per_block(c["output_positions"]))
     assert np.array_equal(got, ref)
-    # worst-case staging selected by max_elems <= 0
-    assert np.array_equal(run_emul(emul, c, max_elems=0, grid=1), ref)
+    # worst-case staging selected by max_elems <= 0; the two-pass fall-back route on every input
+    assert np.array_equal(run_emul(emul, c, max_elems=0, grid=1, two_pass=True), ref)
 
 
 @pytest.mark.parametrize("kind", ["normal", "zeros", "fib", "uniform256"])
@@ -136,9 +137,10 @@ def test_emulated_kernel_small_staging_is_clamped_not_overrun(emul, tmp_path):
 def test_emulated_kernel_under_asan(emul, tmp_path, kind, n, cm, om):
     w = make_case(kind, n, 53)
     c = compress_product(w)
-    got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
-                   out_misalign=om, tmp_path=tmp_path)
-    assert np.array_equal(got, w)
+    for two_pass in (False, True):
+        got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
+                       out_misalign=om, tmp_path=tmp_path, two_pass=two_pass)
+        assert np.array_equal(got, w)
 
 
 # ---------------------------------------------------------------- derived tables
