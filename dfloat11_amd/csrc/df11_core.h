@@ -251,8 +251,8 @@ DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo
 // replayed into the staging area with no further table access.  A chunk that
 // needs more lookups than there are slots reports `overflow` and is handled by
 // count_chunk / emit_chunk instead.
-constexpr int kMainSlots = 8;
-constexpr int kTailSlots = 3;
+constexpr int kMainSlots = 7;
+constexpr int kTailSlots = 2;
 constexpr int kSlots = kMainSlots + kTailSlots;
 
 struct ChunkSyms {
