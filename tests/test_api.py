@@ -1,0 +1,199 @@
+"""The drop-in Python API: compress_model -> DF11 safetensors -> DFloat11Model.from_pretrained,
+with the reference's names, files and error behaviour (no GPU needed for these)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+from safetensors.torch import load_file
+
+from dfloat11_amd import DFloat11Model, compress_model
+from dfloat11_amd import dfloat11 as M
+
+
+class Block(nn.Module):
+    def __init__(self, d, h):
+        super().__init__()
+        self.attn = nn.Module()
+        self.attn.q_proj = nn.Linear(d, d, bias=False)
+        self.attn.o_proj = nn.Linear(d, d, bias=True)
+        self.mlp = nn.Module()
+        self.mlp.up = nn.Linear(d, h, bias=False)
+        self.mlp.down = nn.Linear(h, d, bias=False)
+        self.norm = nn.LayerNorm(d)
+
+    def forward(self, x):
+        x = x + self.attn.o_proj(self.attn.q_proj(self.norm(x)))
+        return x + self.mlp.down(torch.relu(self.mlp.up(x)))
+
+
+class Tiny(nn.Module):
+    def __init__(self, vocab=97, d=64, h=160, n_layers=3):
+        super().__init__()
+        self.embed = nn.Embedding(vocab, d)
+        self.layers = nn.ModuleList([Block(d, h) for _ in range(n_layers)])
+        self.lm_head = nn.Linear(d, vocab, bias=False)
+
+    def forward(self, ids):
+        x = self.embed(ids)
+        for layer in self.layers:
+            x = layer(x)
+        return self.lm_head(x)
+
+
+PATTERNS = {
+    r"embed": [],
+    r"layers\.\d+": ["attn.q_proj", "attn.o_proj", "mlp.up", "mlp.down"],
+    r"lm_head": [],
+}
+
+
+def make_model(seed=0):
+    torch.manual_seed(seed)
+    m = Tiny().to(torch.bfloat16)
+    with torch.no_grad():
+        for p in m.parameters():
+            if p.dim() > 1:
+                p.copy_((torch.randn(p.shape) * 0.02).to(torch.bfloat16))
+    return m.eval()
+
+
+@pytest.fixture()
+def compressed(tmp_path):
+    model = make_model()
+    originals = {k: v.clone() for k, v in model.state_dict().items()}
+    compress_model(model, PATTERNS, str(tmp_path), check_correctness=False)
+    return tmp_path, originals
+
+
+def test_files_and_config(compressed):
+    path, originals = compressed
+    assert sorted(os.listdir(path)) == ["config.json", "model.safetensors"]
+    cfg = json.load(open(path / "config.json"))["dfloat11_config"]
+    assert cfg == {"version": "0.5.0", "threads_per_block": [512], "bytes_per_thread": 8,
+                   "pattern_dict": PATTERNS}
+    tensors = load_file(str(path / "model.safetensors"))
+    for mod in ("embed", "layers.0", "layers.2", "lm_head"):
+        for name, dtype in (("luts", torch.uint8), ("encoded_exponent", torch.uint8),
+                            ("sign_mantissa", torch.uint8), ("output_positions", torch.uint8),
+                            ("gaps", torch.uint8), ("split_positions", torch.int64)):
+            assert tensors[f"{mod}.{name}"].dtype == dtype
+    assert "layers.0.attn.q_proj.weight" not in tensors and "embed.weight" not in tensors
+    assert "layers.0.attn.o_proj.bias" in tensors and "layers.1.norm.weight" in tensors
+    # a block stores its four weights as ONE stream, split points between them
+    assert tensors["layers.1.split_positions"].tolist() == [64 * 64, 2 * 64 * 64, 2 * 64 * 64 + 160 * 64]
+    assert tensors["embed.split_positions"].numel() == 0
+    n = 2 * 64 * 64 + 2 * 160 * 64
+    assert tensors["layers.1.sign_mantissa"].numel() == n
+    n_blocks = -(-tensors["layers.1.encoded_exponent"].numel() // 4096)
+    assert tensors["layers.1.gaps"].numel() == 320 * n_blocks
+    assert tensors["layers.1.output_positions"].numel() == 4 * (n_blocks + 1)
+    assert tensors["layers.1.luts"].shape[1] == 256
+
+
+def test_streams_decode_to_the_original_weights(compressed, oracle):
+    """What compress_model wrote, read back with the oracle's restatement of the reference kernel."""
+    path, originals = compressed
+    t = load_file(str(path / "model.safetensors"))
+    for mod, names in (("embed", ["embed.weight"]), ("lm_head", ["lm_head.weight"]),
+                       ("layers.2", [f"layers.2.{a}.weight" for a in PATTERNS[r"layers\.\d+"]])):
+        out = oracle.c_decode(t[f"{mod}.luts"].numpy(), t[f"{mod}.encoded_exponent"].numpy(),
+                              t[f"{mod}.sign_mantissa"].numpy(), t[f"{mod}.output_positions"].numpy(),
+                              t[f"{mod}.gaps"].numpy())
+        want = torch.cat([originals[n].flatten() for n in names]).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(out, want)
+
+
+def test_loader_installs_hooks_and_drops_weights(compressed):
+    path, originals = compressed
+    model = DFloat11Model.from_pretrained(str(path), device="cpu", bfloat16_model=make_model(seed=1))
+    for mod in (model.embed, model.layers[0], model.lm_head):
+        assert len(mod._forward_pre_hooks) == 1
+        assert mod.luts.dtype == torch.uint8 and mod.output_positions.dtype == torch.uint8
+        assert isinstance(mod.shared_mem_size, int) and mod.shared_mem_size > 2052
+    assert not hasattr(model.embed, "weight") and not hasattr(model.lm_head, "weight")
+    blk = model.layers[1]
+    assert [type(m) for m in blk.weight_injection_modules] == [nn.Linear] * 4
+    assert not hasattr(blk.attn.q_proj, "weight") and not hasattr(blk.mlp.down, "weight")
+    assert isinstance(blk.split_positions, list) and len(blk.split_positions) == 3
+    # uncompressed tensors were copied into the fresh model
+    assert torch.equal(model.layers[0].attn.o_proj.bias, originals["layers.0.attn.o_proj.bias"])
+    assert torch.equal(model.layers[2].norm.weight, originals["layers.2.norm.weight"])
+
+
+def test_forward_on_cpu_fails_loudly(compressed):
+    path, _ = compressed
+    model = DFloat11Model.from_pretrained(str(path), device="cpu", bfloat16_model=make_model(seed=1))
+    with pytest.raises(RuntimeError, match="GPU"):
+        model(torch.zeros(1, 4, dtype=torch.long))
+
+
+def test_cpu_offload_keeps_streams_on_the_host(compressed):
+    path, _ = compressed
+    model = DFloat11Model.from_pretrained(str(path), device="cpu", bfloat16_model=make_model(seed=1),
+                                          cpu_offload=True, cpu_offload_blocks=2, pin_memory=False)
+    offloaded = [m for m in (model.embed, *model.layers, model.lm_head) if hasattr(m, "offloaded_tensors")]
+    assert len(offloaded) == 2
+    for m in offloaded:
+        assert set(m.offloaded_tensors) == {"encoded_exponent", "sign_mantissa"}
+        assert not hasattr(m, "encoded_exponent") and hasattr(m, "luts") and hasattr(m, "gaps")
+
+
+def test_single_file_and_error_paths(compressed, tmp_path):
+    path, _ = compressed
+    f = str(path / "model.safetensors")
+    model = DFloat11Model.from_single_file(f, pattern_dict=PATTERNS, bfloat16_model=make_model(seed=2), device="cpu")
+    assert hasattr(model.embed, "luts")
+    with pytest.raises(IsADirectoryError):
+        DFloat11Model.from_single_file(str(path), pattern_dict=PATTERNS, bfloat16_model=make_model(), device="cpu")
+    with pytest.raises(FileNotFoundError):
+        DFloat11Model.from_single_file(str(path / "nope.safetensors"), pattern_dict=PATTERNS,
+                                       bfloat16_model=make_model(), device="cpu")
+    # a directory whose config.json lacks dfloat11_config
+    bad = tmp_path / "bad"
+    bad.mkdir()
+    (bad / "config.json").write_text("{}")
+    with pytest.raises(AttributeError, match="dfloat11_config"):
+        DFloat11Model.from_pretrained(str(bad), device="cpu", bfloat16_model=make_model())
+
+
+def test_block_range_and_sharded_save(tmp_path):
+    model = make_model()
+    compress_model(model, PATTERNS, str(tmp_path), block_range=[1, 3], save_single_file=False,
+                   check_correctness=False)
+    files = sorted(os.listdir(tmp_path))
+    # blocks 2 and 3 of the walk (layers.0, layers.1) are written; the walk stops at block 4, so
+    # neither the rest of the model nor config.json is saved by this invocation
+    assert files == ["layers_0.safetensors", "layers_1.safetensors"]
+    t = load_file(str(tmp_path / "layers_1.safetensors"))
+    assert "layers.1.encoded_exponent" in t and "layers.1.attn.o_proj.bias" in t
+
+
+def test_non_bf16_weights_are_rejected(tmp_path):
+    model = make_model().float()
+    with pytest.raises(AssertionError, match="bfloat16"):
+        compress_model(model, PATTERNS, str(tmp_path), check_correctness=False)
+
+
+def test_check_correctness_needs_a_gpu(tmp_path):
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    with pytest.raises(RuntimeError, match="GPU"):
+        compress_model(make_model(), PATTERNS, str(tmp_path), check_correctness=True)
+
+
+def test_tensor_manager_is_grow_only():
+    M.TensorManager.clear()
+    a = M.TensorManager.allocate_bfloat16("cpu", 100)
+    b = M.TensorManager.allocate_bfloat16(torch.device("cpu"), 40)
+    assert a.numel() == 100 and b.numel() == 40 and b.data_ptr() == a.data_ptr()
+    c = M.TensorManager.allocate_bfloat16("cpu", 1000)
+    assert c.numel() == 1000
+    M.TensorManager.clear()
+
+
+def test_unsupported_stream_geometry_is_rejected():
+    with pytest.raises(NotImplementedError):
+        M.get_hook((256, ), 8)

@@ -1,0 +1,80 @@
+"""The drop-in API on a real MI355X: a DF11 model's outputs are bit-identical to the BF16 model's."""
+import os
+
+import pytest
+import torch
+
+from dfloat11_amd import DFloat11Model, compress_model
+from dfloat11_amd import dfloat11 as M
+from tests.test_api import PATTERNS, Tiny, make_model
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _reference_logits(seed, ids):
+    ref = make_model(seed).to(DEV)
+    with torch.no_grad():
+        return ref(ids)
+
+
+@pytest.mark.parametrize("offload", [False, True])
+def test_forward_bit_identical(tmp_path, offload):
+    print(f"case api forward offload={offload}", flush=True)
+    M._prefetcher.reset()
+    compress_model(make_model(3), PATTERNS, str(tmp_path), check_correctness=True, check_device=DEV)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device=DEV, bfloat16_model=make_model(9),
+                                          cpu_offload=offload)
+    ids = torch.randint(0, 97, (4, 16), device=DEV)
+    want = _reference_logits(3, ids)
+    with torch.no_grad():
+        for _ in range(3):                       # later passes run with the prefetch order learnt
+            got = model(ids)
+            assert torch.equal(got, want)
+    # derived workspaces are attributes, not part of the saved state
+    assert not any("_df11" in k for k in model.state_dict())
+    if offload:
+        assert not hasattr(model.layers[0], "encoded_exponent")
+        assert model.layers[0].offloaded_tensors["encoded_exponent"].is_pinned()
+
+
+def test_shared_buffer_is_reused_across_modules(tmp_path):
+    print("case api shared buffer", flush=True)
+    M.TensorManager.clear()
+    compress_model(make_model(4), PATTERNS, str(tmp_path), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device=DEV, bfloat16_model=make_model(9))
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+    with torch.no_grad():
+        model(ids)
+    buf = M.TensorManager._tensors[torch.device(DEV)]
+    biggest = max(2 * 64 * 64 + 2 * 160 * 64, 97 * 64)
+    assert buf.numel() == biggest
+    # every injected weight is a view into that one buffer
+    for lin in model.layers[2].weight_injection_modules:
+        assert buf.data_ptr() <= lin.weight.data_ptr() < buf.data_ptr() + buf.numel() * 2
+
+
+def test_hf_llama_generate_matches_bf16(tmp_path):
+    """transformers path: save_pretrained + AutoConfig, greedy generation token-identical."""
+    print("case api hf llama", flush=True)
+    from transformers import AutoModelForCausalLM, LlamaConfig
+    cfg = LlamaConfig(vocab_size=512, hidden_size=128, intermediate_size=256, num_hidden_layers=3,
+                      num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=128,
+                      tie_word_embeddings=False)
+    torch.manual_seed(0)
+    base = AutoModelForCausalLM.from_config(cfg, torch_dtype=torch.bfloat16).eval()
+    ref = AutoModelForCausalLM.from_config(cfg, torch_dtype=torch.bfloat16).eval()
+    ref.load_state_dict(base.state_dict())
+    patterns = {r"model\.embed_tokens": [], r"lm_head": [],
+                r"model\.layers\.\d+": ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj",
+                                        "self_attn.o_proj", "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj"]}
+    compress_model(base, patterns, str(tmp_path), save_single_file=False, check_correctness=True,
+                   check_device=DEV)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device=DEV)
+    ref = ref.to(DEV)
+    ids = torch.randint(0, 512, (2, 12), device=DEV)
+    with torch.no_grad():
+        assert torch.equal(model(ids).logits, ref(ids).logits)
+        a = model.generate(ids, max_new_tokens=16, do_sample=False)
+        b = ref.generate(ids, max_new_tokens=16, do_sample=False)
+    assert torch.equal(a, b)
