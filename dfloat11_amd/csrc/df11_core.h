@@ -247,8 +247,10 @@ DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo
 // The fast path decodes a chunk once.  The lookups of a chunk are few (each
 // resolves up to four codes), so their results fit in registers: kMainSlots
 // lookups that stay inside the chunk plus kTailSlots for the codes that reach
-// into the look-ahead.  Once the lane's output offset is known, the symbols are
-// replayed into the staging area with no further table access.  A chunk that
+// into the look-ahead (a tail lookup may hold symbols of the next chunk as well:
+// they are the true next symbols of the stream).  Once the lane's output offset
+// is known, the symbols are replayed into the staging area with no further
+// table access.  A chunk that
 // needs more lookups than there are slots reports `overflow` and is handled by
 // count_chunk / emit_chunk instead.
 constexpr int kMainSlots = 7;
@@ -319,27 +321,33 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Luts& l, uint32_t hi,
   return r;
 }
 
-// Write the chunk's r.count symbols to p[0..count).  While four or more bytes
-// remain, a lookup stores its four bytes at once (the bytes past its symbols are
-// zero and are overwritten by the next store); the last one to three symbols are
-// gathered and stored exactly, so nothing is written at or beyond p + count.
-DF11_HD void replay_chunk(const ChunkSyms& r, uint8_t* p) {
-  uint32_t rem = r.count, acc = 0, got = 0;
+// OR a 32-bit value into the aligned word at p.  On the device this is an LDS
+// atomic without return: it costs the same as an aligned store, where a store
+// to an address that is not a multiple of four stalls the LDS pipeline for
+// dozens of cycles.
+DF11_HD void or32_aligned(uint8_t* p, uint32_t v) {
+  uint32_t* w = static_cast<uint32_t*>(__builtin_assume_aligned(p, 4));
+#if defined(__HIP_DEVICE_COMPILE__)
+  __hip_atomic_fetch_or(w, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#else
+  *w |= v;
+#endif
+}
+
+// OR the chunk's symbols into stage[at .. at + r.count), which must hold zeros
+// (`stage` is 4-byte aligned).  Each lookup's four symbol bytes go out as two
+// aligned words, shifted to their byte position; the unused bytes of a lookup
+// are zero and leave their neighbours alone, so no lookup needs trimming and the
+// lanes of a wavefront may write the bytes of one word in any order.
+DF11_HD void replay_chunk(const ChunkSyms& r, uint8_t* stage, uint32_t at) {
+  uint32_t bit = at * 8u;
 #pragma unroll
   for (int i = 0; i < kSlots; ++i) {
-    const uint32_t k = (r.ks >> (3 * i)) & 7u;
-    if (rem >= 4u) {
-      store32(p, r.syms[i]);
-      p += k;
-      rem -= k;
-    } else {
-      acc |= r.syms[i] << got;
-      got += 8u * k;
-    }
-  }
-  if (rem < 4u) {                 // rem == 4 can only be left by a chunk that overflowed its slots
-    if (rem & 2u) store16(p, acc);
-    if (rem & 1u) p[rem & 2u] = (uint8_t)(acc >> (8u * (rem & 2u)));
+    const uint64_t v = (uint64_t)r.syms[i] << (bit & 24u);
+    uint8_t* w = stage + ((bit >> 3) & ~3u);
+    or32_aligned(w, (uint32_t)v);
+    or32_aligned(w + 4, (uint32_t)(v >> 32));
+    bit += ((r.ks >> (3 * i)) & 7u) * 8u;
   }
 }
 
@@ -418,6 +426,14 @@ struct SubPlan {
   uint32_t n_out;   // elements produced (clamped to n_elements and to the staging capacity)
 };
 
+// Staging bytes one wavefront needs for sub-blocks of up to max_sub elements: the
+// output phase (up to 7), the elements, and the 8 bytes that the word pair of a
+// replayed lookup may cover past the last element; a multiple of 16.
+constexpr int kStageSlack = 8;
+DF11_HD int32_t stage_capacity(int32_t max_sub) {
+  return ((max_sub + (kGroup - 1) + kStageSlack + 15) / 16) * 16;
+}
+
 DF11_HD SubPlan plan_sub(int64_t base, uint32_t total, int64_t n_elements, int32_t stage_cap) {
   SubPlan p;
   p.a0 = base & ~(int64_t)(kGroup - 1);
@@ -425,10 +441,16 @@ DF11_HD SubPlan plan_sub(int64_t base, uint32_t total, int64_t n_elements, int32
   int64_t end = base + (int64_t)total;
   if (end > n_elements) end = n_elements;
   int64_t n_out = end > base ? end - base : 0;
-  const int64_t room = (int64_t)stage_cap - (int64_t)p.phase;
+  const int64_t room = (int64_t)stage_cap - kStageSlack - (int64_t)p.phase;
   if (n_out > room) n_out = room;
   p.n_out = (uint32_t)n_out;
   return p;
+}
+
+// Staging bytes a sub-block may have touched, a multiple of 8: what has to be
+// zero again before the next sub-block is replayed into the same area.
+DF11_HD uint32_t stage_used(const SubPlan& p) {
+  return (p.phase + p.n_out + (uint32_t)kStageSlack + 7u) & ~7u;
 }
 
 // How many of its `count` codes a thread with exclusive prefix `excl` decodes.

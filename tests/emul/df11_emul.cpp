@@ -94,7 +94,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   if (max_elems_per_sub <= 0 || max_elems_per_sub > kMaxElemsPerSub) max_elems_per_sub = kMaxElemsPerSub;
   const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
   const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
-  const int stage_cap = ((max_elems_per_sub + kGroup + 15) / 16) * 16;
+  const int stage_cap = stage_capacity(max_elems_per_sub);
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
 
   // exact-size copies of everything the kernel may read
@@ -117,6 +117,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   memcpy(rows.p, luts, (size_t)n_rows * 256);
   memcpy(rows.p + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
   Exact<uint8_t> stage((size_t)stage_cap);
+  memset(stage.p, 0, (size_t)stage_cap);   // the kernel clears each wavefront's area once at start
 
   const Tables t{ws.p + kWsTablesOffset + kDecOffset, ws.p + kWsTablesOffset + kCntTailOffset};
   const Luts l{rows.p, n_rows};
@@ -157,7 +158,10 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
       bool replay = all_fit && !force_two_pass;
       for (int lane = 0; lane < kLanes; ++lane)
         replay = replay && thread_quota(excl[lane], count[lane], p.n_out) == count[lane];
-      memset(stage.p, 0xDD, (size_t)stage_cap);
+      // Replay ORs into the staging area: it must be all zero here, which is the
+      // previous sub-block's clear of stage_used() bytes and nothing else.
+      for (int i = 0; i < stage_cap; ++i)
+        if (stage.p[i]) return 8;
       // Lanes run concurrently on the device, so no lane may rely on a later lane
       // repairing what it wrote.  Even sub-blocks write in ascending lane order,
       // odd ones in descending order: a store that strays into a neighbour's
@@ -167,7 +171,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
         const uint32_t quota = thread_quota(excl[lane], count[lane], p.n_out);
         // a lane with nothing to write may hold an out-of-range pointer; it must not use it
         uint8_t* dst = quota ? stage.p + p.phase + excl[lane] : nullptr;
-        if (replay) replay_chunk(regs[lane], dst);
+        if (replay) replay_chunk(regs[lane], stage.p, p.phase + excl[lane]);
         else emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota, dst);
       }
       const SubSpans sp = spans_of(p);
@@ -179,6 +183,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
       } else {
         for (uint32_t i = p.phase; i < p.phase + p.n_out; ++i) stream_element(i, p, stage.p, sm_p, out_p);
       }
+      memset(stage.p, 0, stage_used(p));
     }
   }
   memcpy(out, out_p, (size_t)n_elements * 2);
