@@ -308,7 +308,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   SubInputs cur = fetch_sub(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
   claim(cur.d0, cur.d1, cur.d2, cur.gap_raw, cur.base, cur.end_hint);   // see the claim inside the loop
 
+  // The instruction arbiter prefers the oldest wavefront of a SIMD, so with equal
+  // shares of work the wavefronts launched first would finish well before the
+  // others and leave the CU half empty towards the end.  Each wavefront therefore
+  // walks through the four priority levels, one step every two sub-blocks, from a
+  // starting point given by its slot on the SIMD: over time every wavefront gets
+  // the same share and all of them finish together.
+  uint32_t turn = __builtin_amdgcn_s_getreg((3 << 11) | 4);   // HW_ID.WAVE_ID, the slot on the SIMD
   for (; sub < z.n_subs; sub += stride) {
+    switch ((turn++ >> 1) & 3u) {   // s_setprio takes an immediate
+      case 0: __builtin_amdgcn_s_setprio(0); break;
+      case 1: __builtin_amdgcn_s_setprio(1); break;
+      case 2: __builtin_amdgcn_s_setprio(2); break;
+      default: __builtin_amdgcn_s_setprio(3); break;
+    }
     // ---- requests whose latency the two decode passes hide: the next
     // sub-block's inputs and this one's sign|mantissa bytes
     const int64_t next_sub = sub + stride;
