@@ -78,3 +78,16 @@ def test_hf_llama_generate_matches_bf16(tmp_path):
         a = model.generate(ids, max_new_tokens=16, do_sample=False)
         b = ref.generate(ids, max_new_tokens=16, do_sample=False)
     assert torch.equal(a, b)
+
+
+def test_inference_cli_synthetic_matches_bf16():
+    """The generation benchmark on a small random-init Qwen3-shaped model with tied
+    embeddings: DF11 logits and greedy tokens are bit-identical to BF16's."""
+    print("case api inference cli", flush=True)
+    from dfloat11_amd import inference
+    M._prefetcher.reset()
+    report = inference.main(["--synthetic", "tiny", "--num_tokens", "12", "--batch_size", "3",
+                             "--prompt_len", "9", "--compare_bf16", "--json", "--device", DEV])
+    assert report["logits_bit_identical"] and report["tokens_identical"]
+    assert report["df11"]["new_tokens_per_sequence"] == 12
+    assert 0.5 < report["compressed_over_bf16"] < 0.8
