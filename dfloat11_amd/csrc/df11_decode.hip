@@ -316,12 +316,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   // The instruction arbiter prefers the oldest wavefront of a SIMD, so with equal
   // shares of work the wavefronts launched first would finish well before the
   // others and leave the CU half empty towards the end.  Each wavefront therefore
-  // walks through the four priority levels, one step every two sub-blocks, from a
+  // walks through the four priority levels, one step per sub-block, from a
   // starting point given by its slot on the SIMD: over time every wavefront gets
   // the same share and all of them finish together.
   uint32_t turn = __builtin_amdgcn_s_getreg((3 << 11) | 4);   // HW_ID.WAVE_ID, the slot on the SIMD
   for (; sub < z.n_subs; sub += stride) {
-    switch ((turn++ >> 1) & 3u) {   // s_setprio takes an immediate
+    switch (turn++ & 3u) {   // s_setprio takes an immediate
       case 0: __builtin_amdgcn_s_setprio(0); break;
       case 1: __builtin_amdgcn_s_setprio(1); break;
       case 2: __builtin_amdgcn_s_setprio(2); break;
