@@ -222,6 +222,7 @@ struct DecodeSizes {
 // 4 -> 153 us, 1 -> 145 us for the 218 M element block; the memory system does
 // better with loads and stores interleaved than with long bursts of either.
 constexpr int kPrefetchGroups = 2;
+constexpr int kBatchAlignGroups = 16;   // batches of 64 groups start on multiples of 16 groups (256 B of output)
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
@@ -341,12 +342,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
     const uint32_t first_body = (base != a0) ? 1u : 0u;       // group 0 is a partial head unless aligned
     const uint8_t* sm0 = sign_mantissa + a0;                  // uniform bases
     uint16_t* out0 = out + a0;
+    // Lanes are assigned to groups so that every 64-lane batch starts on a 256-byte
+    // boundary of the output (128 bytes of sign|mantissa): the first `skew` lanes of
+    // the first batch stay idle.  A sub-block starts at an arbitrary element, and
+    // 1 KB stores that straddle lines cost 9 % of the kernel's time on fresh data.
+    const uint32_t skew = ((a0 >> 3) + first_body) & (uint32_t)(kBatchAlignGroups - 1);
     U32x2 m[kPrefetchGroups];
 #pragma unroll
     for (int k = 0; k < kPrefetchGroups; ++k) {
       m[k] = U32x2{0, 0};
-      const uint32_t s0 = (first_body + lane + (uint32_t)(kLanes * k)) * (uint32_t)kGroup;
-      if (vec_ok && s0 + (uint32_t)kGroup <= hint_len) m[k] = load_stream(sm0 + s0);
+      const uint32_t s0 = (first_body + lane + (uint32_t)(kLanes * k) - skew) * (uint32_t)kGroup;
+      if (vec_ok && (k > 0 || lane >= skew) && s0 + (uint32_t)kGroup <= hint_len) m[k] = load_stream(sm0 + s0);
     }
     // The ragged ends, fewer than 8 elements each: lanes 0..7 take the head, lanes
     // 8..15 the tail, one element per lane, its sign|mantissa byte requested now.
@@ -403,11 +409,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
       // sign|mantissa byte of the first kPrefetchGroups x 64 groups and of the ragged
       // ends is in registers.
       U32x4 o[kPrefetchGroups];
-      uint32_t g = sp.body_begin + lane;
+      uint32_t g = sp.body_begin + lane - skew;   // below body_begin (or wrapped) for the idle lanes of batch 0
 #pragma unroll
       for (int k = 0; k < kPrefetchGroups; ++k) {
         const uint32_t gk = g + (uint32_t)(kLanes * k);
-        const uint32_t s0 = (gk < sp.body_end ? gk : 0u) * (uint32_t)kGroup;   // in range for idle lanes too
+        const bool on = (k > 0 || lane >= skew) && gk < sp.body_end;
+        const uint32_t s0 = (on ? gk : 0u) * (uint32_t)kGroup;   // in range for idle lanes too
         o[k] = merge8(load_as<U32x2>(stage + s0), m[k]);
       }
       const bool is_head = lane < (uint32_t)kGroup;
@@ -417,7 +424,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
 #pragma unroll
       for (int k = 0; k < kPrefetchGroups; ++k) {
         const uint32_t gk = g + (uint32_t)(kLanes * k);
-        if (gk < sp.body_end) store_stream(out0 + gk * (uint32_t)kGroup, o[k]);
+        if ((k > 0 || lane >= skew) && gk < sp.body_end) store_stream(out0 + gk * (uint32_t)kGroup, o[k]);
       }
       if (edge_on) out0[edge] = edge_word;
       // the groups past the prefetched ones
