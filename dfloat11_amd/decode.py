@@ -81,6 +81,37 @@ def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, w
     return out
 
 
+def bind(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,
+         max_elems_per_subblock=0):
+    """Checks the tensors of one stream once and returns the argument tuple that
+    launch() passes to df11_decode.  The tuple holds raw addresses: it is valid for
+    as long as these very tensors are alive and unmoved."""
+    _require_cuda(luts=luts, encoded_exponent=encoded_exponent, sign_mantissa=sign_mantissa,
+                  output_positions=output_positions, gaps=gaps, out=out, workspace=workspace)
+    _check_stream_tensors(luts, encoded_exponent, output_positions, gaps)
+    n_elements = sign_mantissa.numel()
+    n_bytes = encoded_exponent.numel()
+    if out.dtype != torch.bfloat16 or out.numel() < n_elements:
+        raise _native.DF11Error("out must be a bfloat16 tensor with at least n_elements elements")
+    if workspace.numel() * workspace.element_size() < workspace_bytes(n_bytes):
+        raise _native.DF11Error("workspace buffer too small")
+    return (luts.data_ptr(), encoded_exponent.data_ptr(), sign_mantissa.data_ptr(),
+            output_positions.data_ptr(), gaps.data_ptr(), out.data_ptr(),
+            luts.shape[0], n_bytes, n_elements, workspace.data_ptr(), int(max_elems_per_subblock))
+
+
+def launch(bound, device):
+    """df11_decode with arguments from bind(), on the current stream of `device`."""
+    lib = _native.hip_lib()
+    if torch.cuda.current_device() == device.index:
+        rc = lib.df11_decode(*bound, torch.cuda.current_stream(device).cuda_stream)
+    else:
+        with torch.cuda.device(device):
+            rc = lib.df11_decode(*bound, torch.cuda.current_stream(device).cuda_stream)
+    if rc:
+        _native.check(rc, "df11_decode")
+
+
 def calibration_copy(src, dst):
     """Streaming copy of known size (profiler byte-counter calibration)."""
     _require_cuda(src=src, dst=dst)

@@ -169,6 +169,16 @@ def get_hook(threads_per_block, bytes_per_thread):
             raise RuntimeError(
                 f'DFloat11 module is on {device}: weights are decoded on the GPU only; move the model to a GPU')
 
+        # Resident streams: the launch arguments and the injected weight views stay
+        # valid while the stream tensors and the device's shared buffer are the very
+        # same objects, so later calls are one library call and nothing else.
+        plan = module.__dict__.get('_df11_plan')
+        if plan is not None and plan[0] is TensorManager._tensors.get(device) \
+                and plan[1] is module._buffers.get('encoded_exponent') \
+                and plan[2] is module._buffers.get('sign_mantissa') and plan[3] is module._buffers.get('luts'):
+            _decode.launch(plan[4], device)
+            return
+
         parity = None
         if hasattr(module, 'offloaded_tensors'):
             fetched, parity = _prefetcher.fetch(module, device)
@@ -181,8 +191,9 @@ def get_hook(threads_per_block, bytes_per_thread):
         n_elements = sign_mantissa.numel()
         reconstructed = TensorManager.allocate_bfloat16(device, n_elements)
         workspace, max_sub = _workspace_for(module, device, encoded_exponent, n_elements)
-        _decode.decode(module.luts, encoded_exponent, sign_mantissa, module.output_positions,
-                       module.gaps, reconstructed, workspace, max_sub)
+        bound = _decode.bind(module.luts, encoded_exponent, sign_mantissa, module.output_positions,
+                             module.gaps, reconstructed, workspace, max_sub)
+        _decode.launch(bound, device)
 
         if isinstance(module, nn.Linear):
             module.weight = reconstructed.view(module.out_features, module.in_features)
@@ -195,6 +206,9 @@ def get_hook(threads_per_block, bytes_per_thread):
 
         if parity is not None:
             _prefetcher.after_decode(module, device, parity)
+        else:
+            object.__setattr__(module, '_df11_plan', (TensorManager._tensors.get(device), encoded_exponent,
+                                                      sign_mantissa, module.luts, bound))
 
     return decode_hook
 
