@@ -284,6 +284,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   uint8_t* lds_tables = lds;
   uint8_t* lds_rows = lds + kTablesBytes;
   uint8_t* stage = lds_rows + (kMaxDecodeRows + 1) * 256 + wave * (uint32_t)z.stage_cap;
+  const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
+  // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
+  // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
+  // its window starts one byte early and never reaches past them.
+  const uint32_t gap_bit = lane * 5u;
+  const uint32_t gap_byte = min(gap_bit >> 3, (uint32_t)(kLanes * 5 / 8 - 2));
+  const uint32_t gap_shift = 11u - (gap_bit - 8u * gap_byte);
+  int64_t sub = (int64_t)blockIdx.x * kWavesPerGroup + wave;   // uniform
+  const uint32_t vzero = opaque_vector_zero();
+  // The first sub-block's inputs are requested before the tables are copied, so
+  // that their latency overlaps with that of the copy.
+  SubInputs cur{};
+  if (sub < z.n_subs) cur = fetch_sub(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
   {
     const uint4* src = reinterpret_cast<const uint4*>(ws + kWsTablesOffset);
     uint4* dst = reinterpret_cast<uint4*>(lds_tables);
@@ -297,21 +310,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
 
   const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
   const Luts l{lds_rows, n_rows};
-  const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
   const bool vec_ok = z.vec_ok != 0;
   const int64_t stride = (int64_t)gridDim.x * kWavesPerGroup;
-
-  // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
-  // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
-  // its window starts one byte early and never reaches past them.
-  const uint32_t gap_bit = lane * 5u;
-  const uint32_t gap_byte = min(gap_bit >> 3, (uint32_t)(kLanes * 5 / 8 - 2));
-  const uint32_t gap_shift = 11u - (gap_bit - 8u * gap_byte);
-
-  int64_t sub = (int64_t)blockIdx.x * kWavesPerGroup + wave;   // uniform
   if (sub >= z.n_subs) return;
-  const uint32_t vzero = opaque_vector_zero();
-  SubInputs cur = fetch_sub(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
   claim(cur.d0, cur.d1, cur.d2, cur.gap_raw, cur.base, cur.end_hint);   // see the claim inside the loop
 
   // The instruction arbiter prefers the oldest wavefront of a SIMD, so with equal
