@@ -144,8 +144,8 @@ def main():
     # steps decode them in turn, into one output buffer, the way the blocks of a model
     # follow each other: 4 x 295 MB of compressed input is more than the 256 MB of
     # memory-side cache, so every step reads its input from HBM.  (Decoding one and the
-    # same copy over and over measured 9 % faster before the kernel's batches were
-    # line-aligned; see `same_input_kernel_ms_median` in the result.)
+    # same copy over and over is several per cent faster: `same_input_kernel_ms_median`
+    # in the result.)
     from dfloat11_amd import _native
     lib = _native.hip_lib()
     out = torch.empty(n_elements, dtype=torch.bfloat16, device=dev)

@@ -161,6 +161,32 @@ def test_gpu_side_stream_and_repeat():
     assert np.array_equal(b.view(torch.int16).cpu().numpy().view(np.uint16), w2)
 
 
+def test_gpu_decode_in_a_captured_graph():
+    """df11_decode allocates nothing and never synchronises, so it can be captured into
+    a HIP graph; every replay (with eager work and synchronisation between replays)
+    reproduces the eager result."""
+    print("case graph capture", flush=True)
+    w = make_case("outliers", 400_000, 131)
+    c = compress_product(w)
+    g = to_gpu(c)
+    ws, max_sub = D.prepare(g["luts"], g["encoded_exponent"], g["output_positions"], g["gaps"], w.size)
+    out = torch.zeros(w.size, dtype=torch.bfloat16, device=DEV)
+    args = (g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"], out, ws, max_sub)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        D.decode(*args)                      # warm-up outside the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        D.decode(*args)
+    for _ in range(4):
+        out.fill_(1.0)                       # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), w)
+
+
 def test_gpu_full_size_linear_round_trip():
     """4096x4096 N(0, 0.02): encode -> decode is the identity (size-independent property)."""
     print("case 4096x4096", flush=True)
