@@ -218,3 +218,25 @@ def test_gpu_llama_block_round_trip():
              out, ws, max_sub)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), w.view(torch.int16))
+
+
+@pytest.mark.parametrize("kind", ["outliers", "uniform256", "zeros"])
+def test_gpu_embedding_sized_adversarial_round_trip(kind):
+    """151936 x 4096 (622 329 856 elements) with an adversarial exponent mix: encode ->
+    decode is the identity at the largest tensor size of the Qwen3-8B shape."""
+    print(f"case embedding {kind}", flush=True)
+    import bench_extra
+    w = bench_extra.make_mix(torch, kind, 151936 * 4096, torch.device(DEV), seed=23)
+    from dfloat11_amd import dfloat11_utils as U
+    w_cpu = w.cpu()
+    _, counter = U.get_codec(w_cpu)
+    codec, _, table = U.get_32bit_codec(counter)
+    luts = U.get_luts(table)
+    enc, sm, pos, gaps, _ = U.encode_weights([w_cpu], codec)
+    del w_cpu
+    d = [t.to(DEV) for t in (luts, enc, sm, pos.view(torch.uint8), gaps)]
+    ws, max_sub = D.prepare(d[0], d[1], d[3], d[4], w.numel())
+    out = torch.empty_like(w)
+    D.decode(d[0], d[1], d[2], d[3], d[4], out, ws, max_sub)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), w.view(torch.int16))
