@@ -35,6 +35,47 @@ def _check_stream_tensors(luts, encoded_exponent, output_positions, gaps):
         raise _native.DF11Error("gaps shorter than 320 bytes per bitstream block")
 
 
+def validate_stream(luts, encoded_exponent, sign_mantissa, output_positions, gaps, name="stream"):
+    """Load-time check of one DF11 stream's layout (any device; reads the block
+    positions on the host).  The reference decodes whatever it is given; a stream
+    that fails here would make it read or write out of bounds.  Raises DF11Error."""
+    def bad(why):
+        raise _native.DF11Error(f"{name}: malformed DF11 stream: {why}")
+
+    if luts.dtype != torch.uint8 or luts.dim() != 2 or luts.shape[1] != 256 or luts.shape[0] < 2:
+        bad(f"luts must be uint8 [n_luts >= 2, 256], got {luts.dtype} {tuple(luts.shape)}")
+    if luts.shape[0] - 1 > 17:
+        bad(f"{luts.shape[0] - 1} decode tables, but a pointer entry can name 16 beside the root")
+    for label, t in (("encoded_exponent", encoded_exponent), ("sign_mantissa", sign_mantissa), ("gaps", gaps)):
+        if t.dtype != torch.uint8 or t.dim() != 1:
+            bad(f"{label} must be a flat uint8 tensor")
+    n_bytes, n_elements = encoded_exponent.numel(), sign_mantissa.numel()
+    n_blocks = -(-n_bytes // 4096)
+    if n_elements >= 1 << 32:
+        bad("more than 2^32 - 1 elements in one stream")
+    if n_elements > 8 * n_bytes:
+        bad(f"{n_elements} elements cannot come from {n_bytes} bytes of bitstream")
+    if gaps.numel() != 320 * n_blocks:
+        bad(f"gaps has {gaps.numel()} bytes, expected {320 * n_blocks}")
+    pos = output_positions.detach().cpu().contiguous().view(torch.uint8)
+    if pos.numel() % 4:
+        bad("output_positions is not a whole number of 32-bit words")
+    pos = pos.view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    if pos.numel() not in (n_blocks, n_blocks + 1):
+        bad(f"output_positions has {pos.numel()} entries for {n_blocks} bitstream blocks")
+    if pos.numel():
+        if int(pos[0]) != 0:
+            bad("the first block does not start at element 0")
+        if bool((pos[1:] < pos[:-1]).any()):
+            bad("block positions decrease")
+        if bool((pos[1:] - pos[:-1] > 4096 * 8).any()):
+            bad("a block claims more elements than it has bits")
+        if pos.numel() == n_blocks + 1 and int(pos[-1]) != n_elements:
+            bad(f"last position {int(pos[-1])} differs from the number of elements {n_elements}")
+        if int(pos[-1]) > n_elements:
+            bad("a block starts past the last element")
+
+
 def prepare(luts, encoded_exponent, output_positions, gaps, n_elements, workspace=None):
     """Build the decode workspace of one stream (load time; waits for the current stream).
     Returns (workspace uint8 tensor, max_elems_per_subblock)."""

@@ -144,6 +144,11 @@ def _workspace_for(module, device, encoded_exponent, n_elements):
     """The module's decode workspace on `device`, built on first use there."""
     ws = getattr(module, '_df11_workspace', None)
     if ws is None or ws.device != device:
+        if ws is None:   # first use: check the layout once, before anything is launched on it
+            sign_mantissa = (module.offloaded_tensors['sign_mantissa'] if hasattr(module, 'offloaded_tensors')
+                             else module.sign_mantissa)
+            _decode.validate_stream(module.luts, encoded_exponent, sign_mantissa, module.output_positions,
+                                    module.gaps, type(module).__name__)
         ws, max_sub = _decode.prepare(module.luts, encoded_exponent, module.output_positions,
                                       module.gaps, n_elements)
         # plain attributes, not buffers: derived data must not leak into state_dict()

@@ -197,3 +197,33 @@ def test_tensor_manager_is_grow_only():
 def test_unsupported_stream_geometry_is_rejected():
     with pytest.raises(NotImplementedError):
         M.get_hook((256, ), 8)
+
+
+def test_validate_stream_accepts_good_and_names_what_is_wrong():
+    """Load-time layout check (the reference has none: a malformed stream makes its
+    kernel read or write out of bounds)."""
+    import numpy as np
+    from dfloat11_amd import decode as D
+    from dfloat11_amd._native import DF11Error
+    from tests.df11_cases import compress_product, make_case
+    c = compress_product(make_case("normal", 30_000, 5))
+    t = {k: torch.from_numpy(np.ascontiguousarray(c[k])) for k in
+         ("luts", "encoded_exponent", "sign_mantissa", "gaps")}
+    pos = torch.from_numpy(np.ascontiguousarray(c["output_positions"]).view(np.uint8).copy())
+
+    def check(**over):
+        a = dict(t, output_positions=pos)
+        a.update(over)
+        D.validate_stream(a["luts"], a["encoded_exponent"], a["sign_mantissa"], a["output_positions"], a["gaps"])
+
+    check()
+    check(output_positions=pos[:-4])                      # the reference's own files may lack the final entry
+    bad_pos = pos.clone().view(torch.int32)
+    bad_pos[1] = bad_pos[2] + 1
+    for over, word in ((dict(gaps=t["gaps"][:-1]), "gaps"),
+                       (dict(output_positions=bad_pos.view(torch.uint8)), "decrease"),
+                       (dict(sign_mantissa=t["sign_mantissa"][:-1]), "last position"),
+                       (dict(luts=t["luts"][:1]), "luts"),
+                       (dict(output_positions=pos[:-8]), "entries")):
+        with pytest.raises(DF11Error, match=word):
+            check(**over)
