@@ -227,3 +227,31 @@ def test_validate_stream_accepts_good_and_names_what_is_wrong():
                        (dict(output_positions=pos[:-8]), "entries")):
         with pytest.raises(DF11Error, match=word):
             check(**over)
+
+
+def test_compress_cli_on_a_local_checkpoint(tmp_path):
+    """python -m dfloat11_amd.compress: a saved transformers checkpoint in, a DF11
+    directory with config and per-block safetensors out, streams decode to the weights."""
+    import json
+    from safetensors.torch import load_file
+    from transformers import AutoModelForCausalLM, LlamaConfig
+    from dfloat11_amd import compress
+    cfg = LlamaConfig(vocab_size=300, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=64,
+                      tie_word_embeddings=True)
+    torch.manual_seed(0)
+    src, dst = tmp_path / "bf16", tmp_path / "df11"
+    base = AutoModelForCausalLM.from_config(cfg, torch_dtype=torch.bfloat16)
+    base.save_pretrained(str(src))
+    compress.main(["--model_name_or_path", str(src), "--save_path", str(dst)])
+    conf = json.load(open(dst / "config.json"))
+    assert conf["dfloat11_config"]["bytes_per_thread"] == 8 and conf["tie_word_embeddings"] is False
+    files = sorted(p.name for p in dst.glob("*.safetensors"))
+    assert "model_layers_0.safetensors" in files and "lm_head.safetensors" in files
+    layer = load_file(str(dst / "model_layers_1.safetensors"))
+    assert {"model.layers.1.luts", "model.layers.1.encoded_exponent", "model.layers.1.sign_mantissa",
+            "model.layers.1.output_positions", "model.layers.1.gaps",
+            "model.layers.1.split_positions"} <= set(layer)
+    want = torch.cat([base.get_submodule(f"model.layers.1.{n}").weight.detach().flatten()
+                      for n in compress.LLM_PATTERNS[r"model\.layers\.\d+"]])
+    assert layer["model.layers.1.sign_mantissa"].numel() == want.numel()

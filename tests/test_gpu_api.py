@@ -91,3 +91,24 @@ def test_inference_cli_synthetic_matches_bf16():
     assert report["logits_bit_identical"] and report["tokens_identical"]
     assert report["df11"]["new_tokens_per_sequence"] == 12
     assert 0.5 < report["compressed_over_bf16"] < 0.8
+
+
+def test_compress_cli_output_loads_and_matches(tmp_path):
+    """A tied-embedding checkpoint through `python -m dfloat11_amd.compress`, loaded with
+    DFloat11Model.from_pretrained: logits bit-identical to the BF16 checkpoint's."""
+    print("case api compress cli", flush=True)
+    from transformers import AutoModelForCausalLM, LlamaConfig
+    from dfloat11_amd import compress
+    M._prefetcher.reset()
+    cfg = LlamaConfig(vocab_size=300, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=64,
+                      tie_word_embeddings=True)
+    torch.manual_seed(1)
+    src, dst = tmp_path / "bf16", tmp_path / "df11"
+    AutoModelForCausalLM.from_config(cfg, torch_dtype=torch.bfloat16).save_pretrained(str(src))
+    compress.main(["--model_name_or_path", str(src), "--save_path", str(dst), "--check_correctness"])
+    ref = AutoModelForCausalLM.from_pretrained(str(src), torch_dtype=torch.bfloat16).to(DEV).eval()
+    model = DFloat11Model.from_pretrained(str(dst), device=DEV)
+    ids = torch.randint(0, 300, (2, 11), device=DEV)
+    with torch.no_grad():
+        assert torch.equal(model(ids).logits, ref(ids).logits)
