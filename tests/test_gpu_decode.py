@@ -240,3 +240,30 @@ def test_gpu_embedding_sized_adversarial_round_trip(kind):
     D.decode(d[0], d[1], d[2], d[3], d[4], out, ws, max_sub)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), w.view(torch.int16))
+
+
+def test_gpu_more_than_2_31_elements():
+    """2^31 + 12345 elements in one stream: the reference's kernel indexes with a 32-bit
+    int and stops short of 2^31; here element indices are unsigned 32-bit and byte
+    offsets 64-bit."""
+    print("case above 2^31 elements", flush=True)
+    import bench_extra
+    from dfloat11_amd import dfloat11_utils as U
+    n = (1 << 31) + 12345
+    w = bench_extra.make_mix(torch, "zeros", n, torch.device(DEV), seed=29)
+    w[-5:] = torch.tensor([1.5, -2.0, 0.007, 3e-5, -0.0], dtype=torch.bfloat16, device=DEV)
+    w[n // 2] = 1234.0
+    w_cpu = w.cpu()
+    _, counter = U.get_codec(w_cpu)
+    codec, _, table = U.get_32bit_codec(counter)
+    luts = U.get_luts(table)
+    enc, sm, pos, gaps, _ = U.encode_weights([w_cpu], codec)
+    del w_cpu
+    assert int(pos.view(torch.int32)[-1].item()) & 0xFFFFFFFF == n
+    d = [t.to(DEV) for t in (luts, enc, sm, pos.view(torch.uint8), gaps)]
+    D.validate_stream(d[0], d[1], d[2], d[3], d[4])
+    ws, max_sub = D.prepare(d[0], d[1], d[3], d[4], n)
+    out = torch.empty_like(w)
+    D.decode(d[0], d[1], d[2], d[3], d[4], out, ws, max_sub)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), w.view(torch.int16))
