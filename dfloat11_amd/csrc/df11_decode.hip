@@ -496,7 +496,7 @@ constexpr int kLdsPerCu = 160 * 1024;
 
 // Workgroups resident per CU.  Three (six wavefronts per SIMD) hide the decode
 // latency completely; a fourth only adds memory streams that compete for HBM
-// pages and measured 6 % slower.
+// pages and measured 3 % slower; two are 8 % slower.
 constexpr int kMaxGroupsPerCu = 3;
 int groups_per_cu(size_t lds_bytes) {
   int n = (int)(kLdsPerCu / lds_bytes);
