@@ -63,21 +63,46 @@ DF11_HD void walk(const Luts& l, uint64_t window, uint32_t& sym, uint32_t& len) 
 // ---- table construction (one entry per call) --------------------------------
 
 // Is the code at the top of `window` settled by its first `known` bits alone?
+// If so, returns its symbol and length.  The bits of `window` below the known
+// ones must be zero.
+//
 // The byte LUTs answer for any 8-bit index, including indices whose low bits
-// are not known yet; the answer counts only if it uses no more than the known
-// bits AND does not change when the unknown bits do.  The second condition
-// rejects slots that merely inherited a neighbour's symbol (the end-of-stream
-// code's slots, unused code space): there the symbol found with the unknown
-// bits at 0 and at 1 differs, or its length exceeds the known bits.
+// are not known yet and slots that no code owns (the end-of-stream code's
+// slots, unused code space), which hold whatever the builder of the LUTs filled
+// them with.  The rule below is independent of that filling.  Whole known bytes
+// index slots that a code or a pointer owns (the known bits start a code of the
+// stream).  Where the known bits end inside a byte, the code is settled only if
+// every slot that the unknown bits can select holds the same symbol, and that
+// symbol's recorded length belongs to this level (8*level+1 .. 8*level+8) and
+// fits into the known bits: if the known bits were only the beginning of a
+// longer code, that code's own slots (or the pointer towards it) would lie
+// among the selected ones and either differ from the rest or, when all of them
+// are equal, be an entry longer than the known bits.
 DF11_HD bool resolve(const Luts& l, uint64_t window, uint32_t known, uint32_t& sym, uint32_t& len) {
-  if (known == 0) return false;
-  const uint64_t unknown_mask = known >= 64u ? 0ull : (~0ull >> known);
-  uint32_t s0, n0, s1, n1;
-  walk(l, window & ~unknown_mask, s0, n0);
-  walk(l, window | unknown_mask, s1, n1);
-  sym = s0;
-  len = n0;
-  return n0 <= known && s0 == s1 && n0 == n1;
+  uint32_t row = 0;
+  for (uint32_t level = 0; level <= 3u; ++level) {
+    if (known <= 8u * level) return false;                   // nothing known of this byte
+    const uint32_t kb = known - 8u * level;                  // known bits of this byte, 8 = all
+    const uint32_t lo = (uint32_t)(window >> (56u - 8u * level)) & 0xffu;
+    const uint32_t d = l.rows[row * 256u + lo];
+    if (kb < 8u) {
+      const uint32_t hi = lo | (0xffu >> kb);
+      for (uint32_t j = lo + 1u; j <= hi; ++j)
+        if (l.rows[row * 256u + j] != d) return false;
+    }
+    const uint32_t next_row = 256u - d;
+    if (level < 3u && d >= 240u && next_row < (uint32_t)l.n_rows) {   // a pointer
+      if (kb < 8u) return false;                             // the code continues past the known bits
+      row = next_row;
+      continue;
+    }
+    const uint32_t n = l.rows[(uint32_t)l.n_rows * 256u + d];
+    if (n <= 8u * level || n > 8u * level + 8u) return false;   // not an entry of this level: filling
+    sym = d;
+    len = n;
+    return n <= known;
+  }
+  return false;
 }
 
 DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_t& meta) {

@@ -67,3 +67,106 @@ def compress_product(w_u16):
 def max_elems_per_block(pos):
     pos = np.asarray(pos).astype(np.int64)
     return int((pos[1:] - pos[:-1]).max()) if pos.size > 1 else 0
+
+
+def random_prefix_code(rng):
+    """A random, possibly incomplete prefix code in the DF11 layout, or None when
+    the drawn tree does not fit it (more than 16 sub-tables).  Leaves of a random
+    binary tree of depth <= 32; some leaves stay unused, one is the end-of-stream
+    code, symbols >= 240 only sit on leaves of 25 bits and more."""
+    leaves = [(1, 0), (1, 1)]
+    target = int(rng.choice([2, 3, 4, 6, 10, 20, 40, 80]))
+    deep_bias = rng.random()
+    while len(leaves) < target:
+        if rng.random() < deep_bias:
+            i = int(np.argmax([l for l, _ in leaves]))
+        else:
+            i = int(rng.integers(len(leaves)))
+        l, v = leaves[i]
+        if l >= 32:
+            if all(l2 >= 32 for l2, _ in leaves):
+                break
+            continue
+        leaves[i] = (l + 1, v << 1)
+        leaves.append((l + 1, (v << 1) | 1))
+    rng.shuffle(leaves)
+    n_unused = int(rng.integers(0, max(1, len(leaves) // 2)))
+    used = leaves[: max(2, len(leaves) - n_unused)]
+    eof, used = used[0], used[1:]
+    code_len = np.zeros(256, np.uint8)
+    code_val = np.zeros(256, np.uint32)
+    low = list(rng.permutation(240))
+    high = list(rng.permutation(np.arange(240, 256)))
+    for l, v in used:
+        s = high.pop() if (l >= 25 and high and rng.random() < 0.5) else low.pop()
+        code_len[s], code_val[s] = l, v
+    codec = U.DF11Codec(code_len, code_val, eof[0], eof[1])
+    try:
+        luts = U.get_luts(codec.get_code_table()).numpy()
+    except ValueError:
+        return None
+    return codec, luts
+
+
+def refill_unowned_slots(luts, codec, policy, rng):
+    """The same LUT rows with every slot that no code word and no pointer owns
+    rewritten: 'forward' = rows start at zero and a slot repeats its predecessor,
+    pointers included (the reference builder's forward fill,
+    dfloat11_utils.py:103-106); 'random' = any symbol that has a code or any
+    pointer to an existing row."""
+    code_len, code_val = codec.code_len, codec.code_val
+    n_rows = luts.shape[0] - 1
+    syms = [s for s in range(256) if code_len[s]]
+    prefixes = sorted({(lv, int(code_val[s]) >> (int(code_len[s]) - 8 * lv)) for s in syms
+                       for lv in range((int(code_len[s]) - 1) // 8 + 1)})
+    assert len(prefixes) == n_rows
+    out = luts.copy()
+    for pi, (lv, pv) in enumerate(prefixes):
+        owned = np.zeros(256, bool)
+        for s in syms:
+            l, v = int(code_len[s]), int(code_val[s])
+            if l <= 8 * lv or (v >> (l - 8 * lv)) != pv:
+                continue
+            if (l - 1) // 8 == lv:
+                rem = l - 8 * lv
+                key = (v & ((1 << rem) - 1)) << (8 - rem)
+                owned[key:key + (1 << (8 - rem))] = True
+            else:
+                owned[(v >> (l - 8 * lv - 8)) & 0xFF] = True
+        row = out[pi]
+        if policy == "forward":
+            prev = 0
+            for j in range(256):
+                if owned[j]:
+                    prev = row[j]
+                else:
+                    row[j] = prev
+        elif policy == "random":
+            choices = np.array(syms + [256 - r for r in range(1, n_rows)], dtype=np.uint8)
+            fill = rng.choice(choices, 256)
+            row[~owned] = fill[~owned]
+        else:
+            raise ValueError(policy)
+    return out
+
+
+def random_code_case(seed, max_n=20_000):
+    """(w, streams per fill policy) for a random prefix code, or None."""
+    rng = np.random.default_rng(seed)
+    made = random_prefix_code(rng)
+    if made is None:
+        return None
+    codec, luts = made
+    syms = np.array([s for s in range(256) if codec.code_len[s]], dtype=np.uint8)
+    n = int(np.exp(rng.uniform(0, np.log(max_n))))
+    p = rng.random(syms.size) ** 3 + 1e-6
+    e = rng.choice(syms, n, p=p / p.sum())
+    enc, gaps, pos = U.encode(e, codec)
+    sm = rng.integers(0, 256, n).astype(np.uint8)
+    w = (((sm.astype(np.uint16) & 0x80) << 8) | (e.astype(np.uint16) << 7) | (sm & 0x7F)).astype(np.uint16)
+    cases = {}
+    for policy in ("product", "forward", "random"):
+        l = luts if policy == "product" else refill_unowned_slots(luts, codec, policy, rng)
+        cases[policy] = dict(luts=l, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps,
+                             codec=codec)
+    return w, cases

@@ -9,7 +9,8 @@ import subprocess
 import numpy as np
 import pytest
 
-from tests.df11_cases import KINDS, compress_product, make_case, max_elems_per_block
+from tests.df11_cases import (KINDS, compress_product, make_case, max_elems_per_block,
+                              random_code_case)
 
 EMUL_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
 
@@ -166,22 +167,16 @@ def _first_code(bits, codes):
     return ("void",)
 
 
-@pytest.mark.parametrize("kind,n,seed", [("normal", 300_000, 1), ("outliers", 4097, 61),
-                                         ("outliers", 200_000, 2), ("fib", 330_000, 3),
-                                         ("uniform256", 50_000, 4), ("zeros", 10_000, 5),
-                                         ("high", 3_000, 6), ("single", 100, 7)])
-def test_derived_tables_brute_force(emul, kind, n, seed):
+def _check_tables_against_code(codec, luts):
     """Every entry of the multi-symbol tables against the code table itself: for
     each 11-bit pattern the first (up to four) code words that END inside it,
     and for each shorter pattern the number of code words that START inside it.
     Paths that run into the end-of-stream code or into unused code space are
     exempt from there on: no valid stream contains them before its padding."""
-    c = compress_product(make_case(kind, n, seed))
-    codec = c["codec"]
     codes = {int(s): format(int(codec.code_val[s]), "b").rjust(int(codec.code_len[s]), "0")
              for s in range(256) if codec.code_len[s]}
     codes["eof"] = format(codec.eof_val, "b").rjust(codec.eof_len, "0")
-    dec, cntt = _host_tables(c["luts"])
+    dec, cntt = _host_tables(luts)
     checked = 0
     for idx in range(2048):
         bits = format(idx, "011b")
@@ -216,6 +211,71 @@ def test_derived_tables_brute_force(emul, kind, n, seed):
                 pos += res[2]
             if not void:
                 assert int(cntt[(1 << r) | v]) == starts, (r, bits, int(cntt[(1 << r) | v]), starts)
+
+
+@pytest.mark.parametrize("kind,n,seed", [("normal", 300_000, 1), ("outliers", 4097, 61),
+                                         ("outliers", 200_000, 2), ("fib", 330_000, 3),
+                                         ("uniform256", 50_000, 4), ("zeros", 10_000, 5),
+                                         ("high", 3_000, 6), ("single", 100, 7)])
+def test_derived_tables_brute_force(emul, kind, n, seed):
+    c = compress_product(make_case(kind, n, seed))
+    _check_tables_against_code(c["codec"], c["luts"])
+
+
+@pytest.mark.parametrize("seed", [900, 905, 911, 922, 1059, 1065, 1165, 1195])
+def test_derived_tables_brute_force_random_codes(emul, seed):
+    """Incomplete prefix codes with the unowned LUT slots filled three ways: the
+    tables must not depend on what those slots hold.  (A short code carried into
+    the slots next to a pointer once made an 11-bit prefix of a 26-bit code look
+    like that short code.)"""
+    made = random_code_case(seed, max_n=50)
+    if made is None:
+        pytest.skip("drawn code does not fit the DF11 layout")
+    _, cases = made
+    for policy, c in cases.items():
+        _check_tables_against_code(c["codec"], c["luts"])
+
+
+@pytest.mark.parametrize("chunk", range(8))
+def test_emulated_kernel_random_codes_and_fillings(emul, oracle, chunk):
+    """Random prefix codes (deep, incomplete, symbols >= 240) x three fillings of
+    the unowned LUT slots: kernel == original words, both decode routes.  Where
+    the reference kernel itself could not decode the LUTs (it would spin on a
+    zero-length filling in the stream's padding) only termination is required."""
+    ran = 0
+    for seed in range(1000 + 40 * chunk, 1040 + 40 * chunk):
+        made = random_code_case(seed)
+        if made is None:
+            continue
+        w, cases = made
+        for policy, c in cases.items():
+            try:
+                ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                                      c["output_positions"], c["gaps"])
+            except RuntimeError:
+                run_emul(emul, c)
+                continue
+            assert np.array_equal(ref, w), (seed, policy)
+            for two_pass in (False, True):
+                assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (seed, policy, two_pass)
+            ran += 1
+    assert ran > 20
+
+
+def test_emulated_kernel_few_elements_many_symbols(emul, oracle):
+    """A handful of elements over a large alphabet that includes exponents >= 240:
+    short codes next to 26-bit ones in a stream of a few bytes."""
+    rng = np.random.default_rng(5)
+    for n in (15, 32, 43, 64, 200):
+        syms = np.concatenate([rng.permutation(np.arange(240, 256))[:8], rng.permutation(240)[:190]])
+        e = rng.choice(syms, n).astype(np.uint16)
+        sm = rng.integers(0, 256, n).astype(np.uint16)
+        w = (((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)).astype(np.uint16)
+        c = compress_product(w)
+        ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"], c["output_positions"], c["gaps"])
+        assert np.array_equal(ref, w)
+        for two_pass in (False, True):
+            assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (n, two_pass)
 
 
 @pytest.mark.parametrize("seed", range(60, 72))

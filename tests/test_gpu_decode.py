@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from dfloat11_amd import decode as D
-from tests.df11_cases import KINDS, compress_product, make_case, max_elems_per_block
+from tests.df11_cases import KINDS, compress_product, make_case, max_elems_per_block, random_code_case
 
 pytestmark = pytest.mark.gpu
 
@@ -55,6 +55,37 @@ def test_gpu_matches_oracle(oracle, kind, n):
     got = gpu_decode(c)
     assert np.array_equal(got, ref)
     assert np.array_equal(got, w)
+
+
+def test_gpu_random_codes_and_fillings(oracle):
+    """Random prefix codes (deep, incomplete, symbols >= 240) with the unowned LUT
+    slots filled three ways, and tiny tensors over large alphabets: GPU == original
+    words wherever the reference kernel's restatement can decode the LUTs."""
+    ran = 0
+    for seed in range(2000, 2120):
+        made = random_code_case(seed)
+        if made is None:
+            continue
+        w, cases = made
+        for policy, c in cases.items():
+            try:
+                ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                                      c["output_positions"], c["gaps"])
+            except RuntimeError:
+                continue
+            print(f"case random code seed={seed} filling={policy} n={w.size}", flush=True)
+            assert np.array_equal(ref, w)
+            assert np.array_equal(gpu_decode(c), w), (seed, policy)
+            ran += 1
+    assert ran > 100
+    rng = np.random.default_rng(5)
+    for n in (15, 32, 43, 64, 200):
+        print(f"case few elements, many symbols n={n}", flush=True)
+        syms = np.concatenate([rng.permutation(np.arange(240, 256))[:8], rng.permutation(240)[:190]])
+        e = rng.choice(syms, n).astype(np.uint16)
+        sm = rng.integers(0, 256, n).astype(np.uint16)
+        w = (((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)).astype(np.uint16)
+        assert np.array_equal(gpu_decode(compress_product(w)), w)
 
 
 @pytest.mark.parametrize("kind", ["normal", "zeros", "fib"])
