@@ -365,12 +365,18 @@ int df11_build_luts(const uint8_t code_len[256], const uint32_t code_val[256], u
 
   // Unset entries (the end-of-stream code's slots, unused code space) inherit
   // the most recent symbol entry, carried from row to row; before the first one
-  // that is the symbol with the shortest code.  Any bit pattern, padding
-  // included, therefore decodes to a symbol of non-zero length.
+  // that is the symbol below 240 with the shortest code.  On the first three
+  // levels a decoder reads values of 240 and above as pointers, so only symbols
+  // below 240 may fill there; a code without any (every exponent >= 240) fills
+  // those rows with the row's own first pointer instead.  Any bit pattern,
+  // padding included, therefore decodes to a symbol of non-zero length without
+  // leaving the rows that exist.
   int carried = -1;
-  for (int s = 0; s < kSymbols; ++s)
+  for (int s = 0; s < kPointerFloor; ++s)
     if (code_len[s] && (carried < 0 || code_len[s] < code_len[carried])) carried = s;
-  if (carried < 0) return DF11_ERR_INVALID_ARGUMENT;
+  bool any = false;
+  for (int s = 0; s < kSymbols; ++s) any |= code_len[s] != 0;
+  if (!any) return DF11_ERR_INVALID_ARGUMENT;
 
   for (int pi = 0; pi < n_rows; ++pi) {
     const Prefix& p = prefixes[pi];
@@ -395,9 +401,13 @@ int df11_build_luts(const uint8_t code_len[256], const uint32_t code_val[256], u
       if (entry[key] >= 0 && entry[key] != value) return DF11_ERR_FORMAT;   // not prefix-free
       entry[key] = value;
     }
+    int first_own = -1;
+    for (int i = 0; i < 256 && first_own < 0; ++i) first_own = entry[i];
+    if (first_own < 0) return DF11_ERR_FORMAT;   // a row that no code reaches
     for (int i = 0; i < 256; ++i) {
       if (entry[i] >= 0 && !is_pointer[i]) carried = entry[i];
-      luts[pi * 256 + i] = (uint8_t)(entry[i] >= 0 ? entry[i] : carried);
+      const bool usable = carried >= 0 && (p.level == 3 || carried < kPointerFloor);
+      luts[pi * 256 + i] = (uint8_t)(entry[i] >= 0 ? entry[i] : usable ? carried : first_own);
     }
   }
   std::memcpy(luts + n_rows * 256, code_len, 256);

@@ -146,6 +146,79 @@ def test_reference_decoder_reads_product_streams(oracle, kind, n):
     assert np.array_equal(seq, w)
 
 
+@pytest.mark.parametrize("hist", [{250: 5, 243: 1000}, {250: 5}, {241: 1, 247: 1, 255: 9},
+                                  {s: 1 + s % 7 for s in range(240, 256)}, {250: 5, 241: 7, 100: 3}])
+def test_reference_decoder_reads_streams_of_high_exponents_only(oracle, hist):
+    """With no exponent below 240 there is no symbol that may fill the unowned
+    slots of the first three LUT levels (the reference kernel reads 240..255 there
+    as pointers, decode.cu:105-116): its trailing threads, which decode the padding
+    and the zeros past the stream, must still stay inside the rows that exist."""
+    codec = U.DF11Codec.from_frequencies(hist)
+    luts = U.get_luts(codec.get_code_table()).numpy()
+    n_rows = luts.shape[0] - 1
+    rng = np.random.default_rng(1)
+    e = np.concatenate([np.array(list(hist), np.uint8), rng.choice(np.array(list(hist), np.uint8), 700)])
+    enc, gaps, pos = U.encode(e, codec)
+    sm = rng.integers(0, 256, e.size).astype(np.uint8)
+    w = (((sm.astype(np.uint16) & 0x80) << 8) | (e.astype(np.uint16) << 7) | (sm & 0x7F)).astype(np.uint16)
+    assert np.array_equal(oracle.c_decode(luts, enc, sm, pos, gaps), w)
+    # Rows are ordered by (level, prefix).  On levels 0..2 a value >= 240 must be a
+    # pointer to a row that exists, anything else a symbol that has a code.
+    lens, vals = codec.code_len.astype(int), codec.code_val.astype(int)
+    prefixes = sorted({(lv, vals[s] >> (lens[s] - 8 * lv)) for s in hist for lv in range((lens[s] - 1) // 8 + 1)})
+    assert len(prefixes) == n_rows
+    for r, (level, _) in enumerate(prefixes):
+        for v in luts[r]:
+            if level < 3 and v >= 240:
+                assert 0 < 256 - int(v) < n_rows, (r, int(v))
+            else:
+                assert luts[-1][v] > 0, (r, int(v))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_histograms_build_valid_codes_the_reference_decoder_reads(oracle, seed):
+    """Counts over 50 orders of magnitude, few and many symbols, with and without
+    exponents >= 240: prefix-free, Kraft <= 1, <= 32 bits, high exponents on the
+    fourth level, <= 16 sub-tables, and a round trip through the oracle."""
+    for case in range(60):
+        rng = np.random.default_rng(seed * 1000 + case)
+        k = int(rng.choice([1, 2, 3, 5, 17, 40, 100, 200, 240, 256]))
+        pool = int(rng.integers(0, 3))
+        if pool == 0:
+            syms = rng.permutation(256)[:k]
+        elif pool == 1:
+            syms = rng.permutation(240)[:min(k, 240)]
+        else:
+            hi = rng.permutation(np.arange(240, 256))[:min(k, 16)]
+            syms = np.concatenate([hi, rng.permutation(240)[:max(0, k - hi.size)]])
+        fam = int(rng.integers(0, 4))
+        if fam == 0:
+            cnt = np.floor(2.0 ** rng.uniform(0, 50, syms.size))
+        elif fam == 1:
+            cnt = np.floor(1.618 ** np.arange(syms.size) % 2 ** 52) + 1
+        elif fam == 2:
+            cnt = np.ones(syms.size)
+        else:
+            cnt = np.floor(2.0 ** (np.arange(syms.size) % 45))
+        hist = {int(s): int(c) for s, c in zip(syms, cnt)}
+        codec = U.DF11Codec.from_frequencies(hist)
+        luts = U.get_luts(codec.get_code_table()).numpy()
+        lens = codec.code_len.astype(int)
+        words = sorted([format(int(codec.code_val[s]), "b").rjust(lens[s], "0") for s in hist]
+                       + [format(codec.eof_val, "b").rjust(codec.eof_len, "0")])
+        assert all(not b.startswith(a) for a, b in zip(words, words[1:])), (seed, case)
+        assert sum(2.0 ** -len(x) for x in words) <= 1.0
+        assert lens.max() <= 32 and 0 < codec.eof_len <= 32
+        assert all(lens[s] >= 25 for s in hist if s >= 240)
+        assert luts.shape[0] - 2 <= 16
+        e = np.concatenate([np.array(list(hist), np.uint8), rng.choice(np.array(list(hist), np.uint8), 500)])
+        rng.shuffle(e)
+        enc, gaps, pos = U.encode(e, codec)
+        sm = rng.integers(0, 256, e.size).astype(np.uint8)
+        w = (((sm.astype(np.uint16) & 0x80) << 8) | (e.astype(np.uint16) << 7) | (sm & 0x7F)).astype(np.uint16)
+        assert np.array_equal(oracle.c_decode(luts, enc, sm, pos, gaps), w), (seed, case)
+
+
 def test_fibonacci_reaches_32_bits():
     w = make_case("fib", 400_000, 1)
     c = compress_product(w)
