@@ -76,6 +76,7 @@ class _OffloadPrefetcher:
         self.slots = {}          # (device, parity, name) -> device tensor
         self.pending = {}        # id(module) -> (dict name -> device tensor, copy-done event)
         self.slot_free = {}      # (device, parity) -> event recorded after the last decode that read the slot
+        self.slot_owner = {}     # (device, parity) -> id(module) whose streams the slot holds or is receiving
         self.enabled = True
 
     def _slot(self, device, parity, name, like):
@@ -105,6 +106,20 @@ class _OffloadPrefetcher:
             done = torch.cuda.Event()
             done.record(side)
         self.pending[id(module)] = (tensors, done, parity)
+        self.slot_owner[(device, parity)] = id(module)
+
+    def _prefetched(self, module, device):
+        """True while the copies issued for `module` are still what its slot holds.
+        When modules run in another order than the one learnt (a block skipped, a
+        new one in between), a slot can be handed to another module before the
+        one it was filled for ever runs."""
+        entry = self.pending.get(id(module))
+        if entry is None:
+            return False
+        if self.slot_owner.get((device, entry[2])) != id(module):
+            del self.pending[id(module)]
+            return False
+        return True
 
     def fetch(self, module, device):
         """Device copies of `module`'s offloaded tensors, ready on the current stream."""
@@ -112,7 +127,7 @@ class _OffloadPrefetcher:
         if key not in self.index:
             self.index[key] = len(self.order)
             self.order.append(module)
-        if key not in self.pending:
+        if not self._prefetched(module, device):
             self._issue(module, device)       # first pass, or the prediction missed
         tensors, done, parity = self.pending.pop(key)
         current = torch.cuda.current_stream(device)
@@ -130,7 +145,7 @@ class _OffloadPrefetcher:
         pos = self.index[id(module)]
         if self.enabled and pos + 1 < len(self.order):   # successor known from an earlier pass
             nxt = self.order[pos + 1]
-            if id(nxt) not in self.pending and hasattr(nxt, 'offloaded_tensors'):
+            if hasattr(nxt, 'offloaded_tensors') and not self._prefetched(nxt, device):
                 self._issue(nxt, device)
 
     def reset(self):

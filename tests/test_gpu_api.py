@@ -38,6 +38,30 @@ def test_forward_bit_identical(tmp_path, offload):
         assert model.layers[0].offloaded_tensors["encoded_exponent"].is_pinned()
 
 
+def test_offload_prefetch_survives_a_changing_module_order(tmp_path):
+    """Blocks skipped, run in reverse or twice: the prefetcher's guess of the next
+    module is then wrong, and a staging slot it filled for one module is handed to
+    another before the first ever runs.  Every pass must still decode each
+    module's own streams."""
+    print("case api offload, changing order", flush=True)
+    M._prefetcher.reset()
+    compress_model(make_model(5), PATTERNS, str(tmp_path), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device=DEV, bfloat16_model=make_model(9),
+                                          cpu_offload=True)
+    ref = make_model(5).to(DEV)
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+
+    def run(m, order):
+        x = m.embed(ids)
+        for i in order:
+            x = m.layers[i](x)
+        return m.lm_head(x)
+
+    with torch.no_grad():
+        for order in ([0, 1, 2], [0, 2], [0, 1, 2], [2], [0, 1, 2], [2, 1, 0], [1, 1, 0], [0, 1, 2], [], [0, 1, 2]):
+            assert torch.equal(run(model, order), run(ref, order)), order
+
+
 def test_shared_buffer_is_reused_across_modules(tmp_path):
     print("case api shared buffer", flush=True)
     M.TensorManager.clear()
