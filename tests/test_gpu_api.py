@@ -104,6 +104,30 @@ def test_hf_llama_generate_matches_bf16(tmp_path):
     assert torch.equal(a, b)
 
 
+def test_hf_llama_device_map_auto(tmp_path):
+    """The reference's default call: no device given, device_map='auto' (accelerate
+    places whole compressed blocks; with one GPU everything lands on it)."""
+    print("case api device_map auto", flush=True)
+    from transformers import AutoModelForCausalLM, LlamaConfig
+    cfg = LlamaConfig(vocab_size=384, hidden_size=64, intermediate_size=192, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=64,
+                      tie_word_embeddings=False)
+    torch.manual_seed(1)
+    base = AutoModelForCausalLM.from_config(cfg, torch_dtype=torch.bfloat16).eval()
+    ref = AutoModelForCausalLM.from_config(cfg, torch_dtype=torch.bfloat16).eval()
+    ref.load_state_dict(base.state_dict())
+    patterns = {r"model\.embed_tokens": [], r"lm_head": [],
+                r"model\.layers\.\d+": ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj",
+                                        "self_attn.o_proj", "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj"]}
+    compress_model(base, patterns, str(tmp_path), save_single_file=False, check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path))
+    assert all(b.device.type == "cuda" for b in model.buffers())
+    ref = ref.to(DEV)
+    ids = torch.randint(0, 384, (2, 9), device=DEV)
+    with torch.no_grad():
+        assert torch.equal(model(ids).logits, ref(ids).logits)
+
+
 def test_inference_cli_synthetic_matches_bf16():
     """The generation benchmark on a small random-init Qwen3-shaped model with tied
     embeddings: DF11 logits and greedy tokens are bit-identical to BF16's."""
