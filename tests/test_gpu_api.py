@@ -62,6 +62,28 @@ def test_offload_prefetch_survives_a_changing_module_order(tmp_path):
             assert torch.equal(run(model, order), run(ref, order)), order
 
 
+def test_model_moved_between_cpu_and_gpu(tmp_path):
+    """Loaded on the CPU and moved later, moved away and back (what accelerate's
+    model offload does around every forward): the streams follow the module, the
+    decode binds to the tensors that are there now."""
+    print("case api cpu <-> gpu moves", flush=True)
+    M._prefetcher.reset()
+    compress_model(make_model(6), PATTERNS, str(tmp_path), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device="cpu", bfloat16_model=make_model(9))
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+    want = _reference_logits(6, ids)
+    with pytest.raises(RuntimeError):
+        model(ids.cpu())                      # no CPU decode path
+    with torch.no_grad():
+        model = model.to(DEV)
+        assert torch.equal(model(ids), want)
+        assert torch.equal(model(ids), want)
+        model = model.to("cpu")
+        model = model.to(DEV)
+        assert torch.equal(model(ids), want)
+        assert torch.equal(model(ids), want)
+
+
 def test_shared_buffer_is_reused_across_modules(tmp_path):
     print("case api shared buffer", flush=True)
     M.TensorManager.clear()
