@@ -58,3 +58,13 @@ def test_decode_without_gpu_fails_loudly():
 def test_libraries_are_in_tree():
     assert os.path.dirname(build.HIP_LIB) == os.path.join(ROOT, "dfloat11_amd")
     assert os.path.exists(build.HIP_LIB) and os.path.exists(build.CODEC_LIB)
+
+
+def test_plain_c_caller_builds_against_the_header():
+    """tests/abi/abi_roundtrip.c is C11 compiled by gcc: the header and both
+    libraries are usable without a HIP compiler, Python or torch."""
+    import subprocess
+    d = os.path.join(ROOT, "tests", "abi")
+    subprocess.run(["make", "-s", "-C", d], check=True)
+    out = subprocess.run(["ldd", os.path.join(d, "abi_roundtrip")], capture_output=True, text=True, check=True).stdout
+    assert "libdf11_hip.so" in out and "libdf11_codec.so" in out and "not found" not in out

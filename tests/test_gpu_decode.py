@@ -298,3 +298,15 @@ def test_gpu_more_than_2_31_elements():
     D.decode(d[0], d[1], d[2], d[3], d[4], out, ws, max_sub)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), w.view(torch.int16))
+
+
+@pytest.mark.parametrize("n", [1, 4097, 3_000_001])
+def test_gpu_plain_c_caller_round_trip(n):
+    """The C program of tests/abi: host codec + GPU decode through the C-ABI alone."""
+    print(f"case plain C caller n={n}", flush=True)
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "abi", "abi_roundtrip")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-s", "-C", os.path.dirname(exe)], check=True)
+    res = subprocess.run([exe, str(n)], capture_output=True, text=True, timeout=100)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "mismatches 0" in res.stdout
