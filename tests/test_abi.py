@@ -1,5 +1,4 @@
 """The C-ABI libraries load and export every symbol include/df11.h declares (no GPU calls)."""
-import ctypes
 import os
 import re
 

@@ -1,12 +1,10 @@
 """The drop-in API on a real MI355X: a DF11 model's outputs are bit-identical to the BF16 model's."""
-import os
-
 import pytest
 import torch
 
 from dfloat11_amd import DFloat11Model, compress_model
 from dfloat11_amd import dfloat11 as M
-from tests.test_api import PATTERNS, Tiny, make_model
+from tests.test_api import PATTERNS, make_model
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from dfloat11_amd import decode as D
-from tests.df11_cases import KINDS, compress_product, make_case, max_elems_per_block, random_code_case
+from tests.df11_cases import KINDS, compress_product, make_case, random_code_case
 
 pytestmark = pytest.mark.gpu
 
