@@ -385,7 +385,7 @@ int df11_build_luts(const uint8_t code_len[256], const uint32_t code_val[256], u
     std::fill(entry, entry + 256, -1);
     for (int s = 0; s < kSymbols; ++s) {
       const int l = code_len[s];
-      if (!l || l <= 8 * p.level || (code_val[s] >> (l - 8 * p.level)) != p.value) continue;
+      if (!l || l <= 8 * p.level || (uint32_t)((uint64_t)code_val[s] >> (l - 8 * p.level)) != p.value) continue;   // 64-bit: the shift is 32 for a 32-bit code on level 0
       int key, value;
       if ((l - 1) / 8 == p.level) {
         const int rem = l - 8 * p.level;

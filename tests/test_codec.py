@@ -219,6 +219,24 @@ def test_random_histograms_build_valid_codes_the_reference_decoder_reads(oracle,
         assert np.array_equal(oracle.c_decode(luts, enc, sm, pos, gaps), w), (seed, case)
 
 
+def test_luts_for_a_first_byte_that_only_32_bit_codes_share(oracle):
+    """Codes 0, 1{30 zeros}0 and 1{30 zeros}1: the root row's pointer at 0x80 is
+    owned by 32-bit codes alone (their prefix test shifts by the full word width)."""
+    code_len = np.zeros(256, np.uint8)
+    code_val = np.zeros(256, np.uint32)
+    code_len[7], code_val[7] = 1, 0
+    code_len[9], code_val[9] = 32, 0x80000000
+    code_len[11], code_val[11] = 32, 0x80000001
+    codec = U.DF11Codec(code_len, code_val, 31, 0x40000001)
+    luts = U.get_luts(codec.get_code_table()).numpy()
+    assert luts.shape[0] == 5 and luts[0, 0x80] == 255 and luts[0, 0x7F] == 7
+    e = np.array([7, 9, 7, 7, 11, 11, 9, 7] * 40, np.uint8)
+    enc, gaps, pos = U.encode(e, codec)
+    sm = np.arange(e.size, dtype=np.uint8)
+    w = (((sm.astype(np.uint16) & 0x80) << 8) | (e.astype(np.uint16) << 7) | (sm & 0x7F)).astype(np.uint16)
+    assert np.array_equal(oracle.c_decode(luts, enc, sm, pos, gaps), w)
+
+
 def test_fibonacci_reaches_32_bits():
     w = make_case("fib", 400_000, 1)
     c = compress_product(w)
@@ -241,3 +259,16 @@ def test_encode_rejects_symbol_without_code():
     codec = U.DF11Codec.from_frequencies({5: 10, 6: 3})
     with pytest.raises(ValueError):
         U.encode(np.array([5, 6, 7], np.uint8), codec)
+
+
+def test_codec_under_sanitizers():
+    """tests/emul/df11_codec_san: the host codec built with AddressSanitizer and
+    UndefinedBehaviorSanitizer, random cases plus a Fibonacci histogram with 32-bit
+    codes, each decoded back by the oracle's C restatement."""
+    import os
+    import subprocess
+    d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
+    subprocess.run(["make", "-s", "-C", d, "df11_codec_san"], check=True)
+    res = subprocess.run([os.path.join(d, "df11_codec_san"), "60"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, (res.stdout + res.stderr)[-3000:]
+    assert "0 failures" in res.stdout and "32 bits" in res.stdout
