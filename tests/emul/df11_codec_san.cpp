@@ -1,8 +1,8 @@
 // The host codec (dfloat11_amd/csrc/df11_codec.cpp) under AddressSanitizer and
 // UndefinedBehaviorSanitizer (test infrastructure): random alphabets, skews,
 // sizes and thread counts, and one Fibonacci histogram that reaches 32-bit
-// codes; every stream is decoded back with the oracle's restatement of the
-// reference kernel.  usage: df11_codec_san [cases]
+// codes; every stream is compared with the oracle's restatement of the
+// reference packer and decoded back with its restatement of the reference kernel.  usage: df11_codec_san [cases]
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -15,6 +15,11 @@ extern "C" int df11o_decode_blocks(const uint8_t* luts, const uint8_t* codes, co
                                    const uint32_t* position_offsets, const uint8_t* gaps, uint16_t* outputs,
                                    int n_luts, int64_t n_bytes, int64_t n_elements, int64_t n_positions,
                                    int64_t block_begin, int64_t block_end, int64_t stage_elems);
+
+extern "C" int df11o_encode(const uint8_t* data, int64_t n, const uint8_t* code_len, const uint32_t* code_val,
+                            int eof_len, uint32_t eof_val, uint8_t* encoded, int64_t cap_bytes, int64_t* n_bytes_out,
+                            uint8_t* gaps_packed, int64_t cap_gap_bytes, int64_t* n_gap_bytes_out,
+                            uint32_t* positions, int64_t cap_positions, int64_t* n_positions_out);
 
 static uint64_t state = 88172645463325252ull;
 static uint64_t rnd() {
@@ -44,6 +49,17 @@ static int round_trip(const std::vector<uint16_t>& w, int threads, int* max_len)
   if (df11_encode(e.data(), n, len, val, eof_len, eof_val, enc.data(), n_bytes, gaps.data(), pos.data(), n_blocks,
                   threads))
     return 15;
+  {   // the oracle's restatement of the reference packer writes the same bitstream and gaps
+    std::vector<uint8_t> o_enc(n_bytes + 16), o_gaps(gaps.size() + 640);
+    std::vector<uint32_t> o_pos(n_blocks + 2);
+    int64_t o_nb = 0, o_ng = 0, o_np = 0;
+    if (df11o_encode(e.data(), n, len, val, eof_len, eof_val, o_enc.data(), (int64_t)o_enc.size(), &o_nb,
+                     o_gaps.data(), (int64_t)o_gaps.size(), &o_ng, o_pos.data(), (int64_t)o_pos.size(), &o_np))
+      return 18;
+    if (o_nb != n_bytes || memcmp(o_enc.data(), enc.data(), (size_t)n_bytes)) return 19;
+    if (o_ng != (int64_t)gaps.size() || memcmp(o_gaps.data(), gaps.data(), gaps.size())) return 20;
+    if (o_np < n_blocks || memcmp(o_pos.data(), pos.data(), (size_t)n_blocks * 4)) return 21;
+  }
   std::vector<uint16_t> out(n, 0xEEEE);
   if (df11o_decode_blocks(luts, enc.data(), sm.data(), pos.data(), gaps.data(), out.data(), n_luts, n_bytes, n,
                           n_blocks + 1, 0, n_blocks, DF11_MAX_ELEMS_PER_BLOCK + 1024))
