@@ -191,11 +191,13 @@ def get_hook(threads_per_block, bytes_per_thread):
 
         # Resident streams: the launch arguments and the injected weight views stay
         # valid while the stream tensors and the device's shared buffer are the very
-        # same objects, so later calls are one library call and nothing else.
+        # same objects and nobody has put another `weight` in place of a view, so
+        # later calls are one library call and nothing else.
         plan = module.__dict__.get('_df11_plan')
         if plan is not None and plan[0] is TensorManager._tensors.get(device) \
                 and plan[1] is module._buffers.get('encoded_exponent') \
-                and plan[2] is module._buffers.get('sign_mantissa') and plan[3] is module._buffers.get('luts'):
+                and plan[2] is module._buffers.get('sign_mantissa') and plan[3] is module._buffers.get('luts') \
+                and all(owner.__dict__.get('weight') is view for owner, view in plan[5]):
             _decode.launch(plan[4], device)
             return
 
@@ -217,18 +219,22 @@ def get_hook(threads_per_block, bytes_per_thread):
 
         if isinstance(module, nn.Linear):
             module.weight = reconstructed.view(module.out_features, module.in_features)
+            injected = [(module, module.weight)]
         elif isinstance(module, nn.Embedding):
             module.weight = reconstructed.view(module.num_embeddings, module.embedding_dim)
+            injected = [(module, module.weight)]
         else:
+            injected = []
             weights = torch.tensor_split(reconstructed, module.split_positions)
             for sub_module, weight in zip(module.weight_injection_modules, weights):
                 sub_module.weight = weight.view(sub_module.out_features, sub_module.in_features)
+                injected.append((sub_module, sub_module.weight))
 
         if parity is not None:
             _prefetcher.after_decode(module, device, parity)
         else:
             object.__setattr__(module, '_df11_plan', (TensorManager._tensors.get(device), encoded_exponent,
-                                                      sign_mantissa, module.luts, bound))
+                                                      sign_mantissa, module.luts, bound, injected))
 
     return decode_hook
 

@@ -82,6 +82,25 @@ def test_model_moved_between_cpu_and_gpu(tmp_path):
         assert torch.equal(model(ids), want)
 
 
+def test_replaced_weight_attribute_is_reinjected(tmp_path):
+    """As in the reference, every forward puts the decoded weights back in place
+    (dfloat11.py:153-166), also after someone assigned another tensor to `weight`."""
+    print("case api weight replaced", flush=True)
+    M._prefetcher.reset()
+    compress_model(make_model(7), PATTERNS, str(tmp_path), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device=DEV, bfloat16_model=make_model(9))
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+    want = _reference_logits(7, ids)
+    with torch.no_grad():
+        assert torch.equal(model(ids), want)
+        assert torch.equal(model(ids), want)          # second call: launch arguments already bound
+        lin = model.layers[1].mlp.up
+        lin.weight = torch.zeros_like(lin.weight)
+        model.lm_head.weight = torch.ones_like(model.lm_head.weight)
+        assert torch.equal(model(ids), want)
+        assert torch.equal(model(ids), want)
+
+
 def test_shared_buffer_is_reused_across_modules(tmp_path):
     print("case api shared buffer", flush=True)
     M.TensorManager.clear()
