@@ -87,7 +87,8 @@ DF11_HD bool resolve(const Luts& l, uint64_t window, uint32_t known, uint32_t& s
     const uint32_t d = l.rows[row * 256u + lo];
     if (kb < 8u) {
       const uint32_t hi = lo | (0xffu >> kb);
-      for (uint32_t j = lo + 1u; j <= hi; ++j)
+      if (l.rows[row * 256u + hi] != d) return false;          // the usual way out for an unsettled code
+      for (uint32_t j = lo + 1u; j < hi; ++j)
         if (l.rows[row * 256u + j] != d) return false;
     }
     const uint32_t next_row = 256u - d;
