@@ -42,9 +42,10 @@ def make_block(torch, device):
     return torch.cat(parts)
 
 
-def cpu_baseline(stream, budget_s=12.0):
+def cpu_baseline(stream, original_u16, budget_s=12.0):
     """Times the CPU oracle (scalar C restatement of the reference kernel) on a bounded
-    run of consecutive bitstream blocks of the same stream, on the host's cores."""
+    run of consecutive bitstream blocks of the same stream, on the host's cores, and
+    compares what it decoded with the original BF16 words."""
     from oracle import df11_oracle as O
     n_bytes = stream["encoded_exponent"].size
     n_blocks = -(-n_bytes // 4096)
@@ -79,13 +80,39 @@ def cpu_baseline(stream, budget_s=12.0):
     elems = int(pos[min(sample, pos.size - 1)] - pos[0])
     bytes_done = sample * (4096 + 320 + 4) + 3 * elems
     single = bytes_done / (sample * per_block_1t)
+    first, last = int(pos[0]), int(pos[min(sample, pos.size - 1)])
+    bit_exact = bool(np.array_equal(out[first:last], original_u16[first:last]))
     return {
         "value": bytes_done / dt / 1e9, "unit": "GB/s", "cores": n_threads, "kind": "port",
+        "bit_exact": bit_exact,
         "sample": f"first {sample} of {n_blocks} bitstream blocks of the same stream ({elems} elements), "
                   f"median of {repeats} passes of {dt:.2f} s, scalar C restatement of the reference "
                   f"kernel, one thread per core over disjoint block ranges",
         "single_thread_GBps": single / 1e9,
     }
+
+
+def side_measurements(torch, dev, steps=30, warmup=30):
+    """Kernel-time throughput of the same entry point on other inputs: the 4096x14336
+    matrix under each adversarial exponent distribution, and N(0, 0.02) tensors of the
+    sizes a per-Linear compression produces.  Returns (mixes, sizes): name -> figures."""
+    import bench_extra
+    keep = ("n_elements", "kernel_ms_median", "GBps", "hbm_frac", "bit_exact", "bits_per_exponent",
+            "max_code_bits", "compressed_over_bf16")
+    mixes, sizes = {}, {}
+    for kind in ("laplace", "outliers", "uniform256", "zeros"):
+        w = bench_extra.make_mix(torch, kind, 4096 * 14336, dev, seed=7)
+        r = bench_extra.time_decode(torch, w, steps, warmup)
+        mixes[f"{kind} 4096x14336"] = {k: r[k] for k in keep}
+        del w
+    for rows, cols in ((4096, 4096), (4096, 14336)):
+        g = torch.Generator(device=dev).manual_seed(0)
+        w = (torch.randn(rows * cols, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        r = bench_extra.time_decode(torch, w, steps, warmup)
+        sizes[f"normal {rows}x{cols}"] = {k: r[k] for k in keep}
+        del w
+    torch.cuda.empty_cache()
+    return mixes, sizes
 
 
 def profiled_traffic():
@@ -109,6 +136,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--preheat-ms", type=float, default=400.0,
+                    help="decode launches for this long before the counted warm-up, so that the timed steps "
+                         "run at the clock the device settles at under load, whatever --warmup is")
+    ap.add_argument("--no-mixes", action="store_true",
+                    help="skip the per-distribution and per-size side measurements (config.mixes, config.sizes)")
     ap.add_argument("--copies", type=int, default=4,
                     help="device copies of the compressed block that the steps decode in turn")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -151,11 +183,19 @@ def main():
     out = torch.empty(n_elements, dtype=torch.bfloat16, device=dev)
     stream_handle = torch.cuda.current_stream(dev).cuda_stream
     copies = []
+    prepare_ms = []
     for _ in range(max(1, a.copies)):
         d_luts, d_enc, d_sm, d_gaps = (t.to(dev) for t in (luts, enc, sm, gaps))
         d_pos = pos.view(torch.uint8).to(dev)
-        # load-time step: decode tables and sub-block positions (not part of a decode)
-        ws, max_sub = D.prepare(d_luts, d_enc, d_pos, d_gaps, n_elements)
+        # load-time step, once per compressed module: layout check on the host, then decode
+        # tables and sub-block positions on the device (not part of a decode)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        D.validate_stream(d_luts, d_enc, d_sm, d_pos, d_gaps)
+        t1 = time.perf_counter()
+        ws, max_sub = D.prepare(d_luts, d_enc, d_pos, d_gaps, n_elements)   # waits for its kernels
+        t2 = time.perf_counter()
+        prepare_ms.append(((t1 - t0) * 1e3, (t2 - t1) * 1e3))
         D.decode(d_luts, d_enc, d_sm, d_pos, d_gaps, out, ws, max_sub)   # once through the checked wrapper
         # One step = one call of the C-ABI entry point on torch's current stream, with the
         # arguments bound once (the Python wrapper's checks stay out of the timed region).
@@ -171,6 +211,15 @@ def main():
         if rc != 0:
             raise RuntimeError(f"df11_decode failed: {rc}")
 
+    # Pre-heat by time: the first launches after idle run at a lower clock (about 60 launches
+    # on this device); the counted warm-up follows.
+    t0 = time.perf_counter()
+    preheat_launches = 0
+    while (time.perf_counter() - t0) * 1e3 < a.preheat_ms:
+        for _ in range(16):
+            step()
+        preheat_launches += 16
+        torch.cuda.synchronize()
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
@@ -237,16 +286,34 @@ def main():
             "kernel_ms_min": float(np.min(kernel_ms)), "kernel_ms_max": float(np.max(kernel_ms)),
             "kernel_ms_median": float(np.median(kernel_ms)),
             "input_copies_decoded_in_turn": len(copies), "same_input_kernel_ms_median": same_ms,
+            "preheat_ms": a.preheat_ms, "preheat_launches": preheat_launches,
+            # first-use cost of a compressed module (median over the copies; the first call also
+            # loads the library's code object): host-side layout check + df11_prepare incl. its wait
+            "prepare_ms": float(np.median([v + p for v, p in prepare_ms])),
+            "prepare_ms_validate_stream": float(np.median([v for v, _ in prepare_ms])),
+            "prepare_ms_df11_prepare": float(np.median([p for _, p in prepare_ms])),
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": profiled_traffic(),
                      "kernel": "decode_kernel", "avg_launch_ms": avg_kernel_ms},
     }
+    if not a.no_mixes:
+        copies.clear()
+        out = None
+        torch.cuda.empty_cache()
+        result["config"]["mixes"], result["config"]["sizes"] = side_measurements(torch, dev)
+        if not all(m["bit_exact"] for m in list(result["config"]["mixes"].values())
+                   + list(result["config"]["sizes"].values())):
+            result["error"] = "a side measurement did not decode bit-exactly"
+            bit_exact = False
     if not a.no_cpu_baseline:
         stream = dict(luts=luts.numpy(), encoded_exponent=enc.numpy(), sign_mantissa=sm.numpy(),
                       output_positions=pos.numpy(), gaps=gaps.numpy())
-        result["cpu_baseline"] = cpu_baseline(stream)
-    if bit_exact is False:
+        result["cpu_baseline"] = cpu_baseline(stream, w_cpu.view(torch.int16).numpy().view(np.uint16))
+        if not result["cpu_baseline"]["bit_exact"]:
+            result["error"] = "the CPU oracle's output differs from the original block"
+            bit_exact = False
+    if bit_exact is False and "error" not in result:
         result["error"] = "decoded block differs from the original"
     print(json.dumps(result))
     if bit_exact is False:

@@ -218,7 +218,10 @@ def build_flux(torch, hidden, n_double, n_single, heads, device, seed):
     return model.eval().requires_grad_(False)
 
 
-def run_flux(a, torch, dev):
+def flux_report(a, torch, dev, passes=8):
+    """Runs the FLUX-shaped stack in BF16, with resident DF11 streams and with offloaded
+    DF11 streams; returns the report dict (a: double_blocks, single_blocks, image_tokens,
+    text_tokens)."""
     from dfloat11_amd import dfloat11 as M
     from dfloat11_amd.inference import convert_in_memory
     hidden, heads = 3072, 24
@@ -228,7 +231,7 @@ def run_flux(a, torch, dev):
     c = torch.randn(1, a.text_tokens, hidden, generator=g, device=dev).to(torch.bfloat16)
     temb = torch.randn(1, 1, hidden, generator=g, device=dev).to(torch.bfloat16)
 
-    def timed(model, label, passes=8):
+    def timed(model, label):
         M._prefetcher.reset()
         M.TensorManager.clear()
         torch.cuda.empty_cache()
@@ -309,6 +312,11 @@ def run_flux(a, torch, dev):
         "outputs_bit_identical": {"resident_vs_bf16": bool(torch.equal(y_res, y_ref)),
                                   "offload_vs_resident": bool(torch.equal(y_off, y_res))},
     }
+    return report
+
+
+def run_flux(a, torch, dev):
+    report = flux_report(a, torch, dev)
     print(json.dumps(report), flush=True)
     return all(report["outputs_bit_identical"].values())
 

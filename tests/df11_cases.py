@@ -170,3 +170,37 @@ def random_code_case(seed, max_n=20_000):
         cases[policy] = dict(luts=l, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps,
                              codec=codec)
     return w, cases
+
+
+def short_positions_case(oracle, seed, n_full_blocks):
+    """A stream laid out by the oracle's restatement of the reference encoder whose
+    output_positions comes out one entry short: the last code starts in block
+    n_full_blocks - 1, crosses into the next block and ends on a byte boundary, so the
+    end-of-stream branch that would note the new block is skipped
+    (dfloat11_utils.py:146-162).  The code table is built from a longer run of the same
+    data, then the run is cut and its last exponent chosen so that the quirk occurs.
+    Returns (w, stream dict) with n_full_blocks + 1 bitstream blocks and as many positions."""
+    rng = np.random.default_rng(seed)
+    n = 60_000 * n_full_blocks
+    p = 0.93 ** np.arange(120)
+    e = (rng.choice(120, n, p=p / p.sum()) + 60).astype(np.uint8)
+    _, table = oracle.get_32bit_codec(oracle.get_counter(e))
+    luts = oracle.get_luts(table)
+    lens = luts[-1].astype(np.int64)
+    by_len = {int(lens[s]): s for s in range(256) if lens[s]}
+    cum = np.cumsum(lens[e])
+    boundary = 32768 * n_full_blocks
+    i = int(np.searchsorted(cum, boundary))
+    while True:
+        d = boundary - (int(cum[i - 1]) if i else 0)   # bits left in the block before element i
+        if d >= 1 and (d + 8) in by_len:
+            break
+        i -= 1
+    e = e[: i + 1].copy()
+    e[i] = by_len[d + 8]                               # ends 8 bits into the next block
+    sm = rng.integers(0, 256, e.size).astype(np.uint8)
+    enc, gaps, pos = oracle.c_encode(e, table)
+    n_blocks = -(-enc.size // 4096)
+    assert n_blocks == n_full_blocks + 1 and pos.size == n_blocks and int(pos[-1]) == e.size
+    w = oracle.merge_bf16(e, sm)
+    return w, dict(luts=luts, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps)

@@ -123,6 +123,16 @@ def test_emulated_kernel_short_positions_quirk(emul, oracle):
     assert np.array_equal(run_emul(emul, c), oracle.merge_bf16(data, sm))
 
 
+@pytest.mark.parametrize("seed,n_full", [(1, 1), (2, 3), (3, 9)])
+def test_emulated_kernel_short_positions_multi_block(emul, oracle, seed, n_full):
+    """Realistic code lengths, several blocks, positions one entry short."""
+    from tests.df11_cases import short_positions_case
+    w, c = short_positions_case(oracle, seed, n_full)
+    ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"], c["output_positions"], c["gaps"])
+    assert np.array_equal(ref, w)
+    assert np.array_equal(run_emul(emul, c), w)
+
+
 def test_emulated_kernel_small_staging_is_clamped_not_overrun(emul, tmp_path):
     """A caller that understates max_elems_per_block loses elements but never
     writes outside the staging area (checked under AddressSanitizer)."""

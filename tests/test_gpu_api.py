@@ -199,3 +199,63 @@ def test_compress_cli_output_loads_and_matches(tmp_path):
     ids = torch.randint(0, 300, (2, 11), device=DEV)
     with torch.no_grad():
         assert torch.equal(model(ids).logits, ref(ids).logits)
+
+
+def test_qwen3_8b_shape_generate_matches_bf16():
+    """The full Qwen3-8B shape (36 layers, hidden 4096, MLP 12288, vocabulary 151936, tied
+    embeddings; 7.57 B parameters, random-init N(0, 0.02)): prompt logits and greedy tokens
+    of the DF11 model are bit-identical to the BF16 model's, at batch 1 and batch 64
+    (what the reference checks per block at compression time, dfloat11.py:560-591, here
+    end to end through the hooks)."""
+    print("case api qwen3-8b full shape", flush=True)
+    from dfloat11_amd import inference
+    M._prefetcher.reset()
+    M.TensorManager.clear()
+    dev = torch.device(DEV)
+    model = inference.build_synthetic("qwen3-8b", dev, seed=42)
+    assert sum(p.numel() for p in model.parameters()) == 7_568_405_504
+    batches = {}
+    for batch in (1, 64):
+        gen = torch.Generator(device="cpu").manual_seed(42 + batch)
+        ids = torch.randint(0, model.config.vocab_size, (batch, 64), generator=gen).to(dev)
+        inputs = {"input_ids": ids, "attention_mask": torch.ones_like(ids)}
+        with torch.no_grad():
+            logits = model(**inputs, use_cache=False).logits
+            tokens = model.generate(**inputs, max_new_tokens=8, min_new_tokens=8, do_sample=False)
+        batches[batch] = (inputs, logits, tokens)
+    print("case api qwen3-8b full shape: compressing", flush=True)
+    compressed, original = inference.convert_in_memory(model, inference.LLM_PATTERNS, dev)
+    assert 0.6 < compressed / original < 0.75
+    torch.cuda.empty_cache()
+    assert not any(name.endswith("proj.weight") for name, _ in model.named_parameters())
+    for batch, (inputs, logits, tokens) in batches.items():
+        print(f"case api qwen3-8b full shape: DF11 batch {batch}", flush=True)
+        with torch.no_grad():
+            got_logits = model(**inputs, use_cache=False).logits
+            got_tokens = model.generate(**inputs, max_new_tokens=8, min_new_tokens=8, do_sample=False)
+        assert torch.equal(got_logits, logits), batch
+        assert torch.equal(got_tokens, tokens), batch
+    del model, batches
+    M.TensorManager.clear()
+    torch.cuda.empty_cache()
+
+
+def test_flux_shaped_offloaded_pass_is_bit_identical():
+    """FLUX.1-dev block shapes (hidden 3072, 24 heads, MLP ratio 4; module names and the
+    order of the linears as in the reference's FLUX pattern_dict,
+    examples/compress_flux1/compress_flux.py:49-74), two double-stream and three
+    single-stream blocks, 4096 image + 512 text tokens: the pass with the compressed
+    streams in pinned host memory, copied one block ahead, gives the same bits as the
+    pass with resident streams and as BF16."""
+    print("case api flux-shaped offload", flush=True)
+    import types
+    import bench_extra
+    a = types.SimpleNamespace(double_blocks=2, single_blocks=3, image_tokens=4096, text_tokens=512)
+    report = bench_extra.flux_report(a, torch, torch.device(DEV), passes=4)
+    assert report["config"]["parameters"] == 2 * 339_738_624 + 3 * 141_557_760
+    assert report["outputs_bit_identical"] == {"resident_vs_bf16": True, "offload_vs_resident": True}
+    off, res = report["passes"]["df11_offload"], report["passes"]["df11_resident"]
+    assert off["peak_device_memory_mb"] < res["peak_device_memory_mb"]
+    M._prefetcher.reset()
+    M.TensorManager.clear()
+    torch.cuda.empty_cache()

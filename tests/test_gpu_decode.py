@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from dfloat11_amd import decode as D
-from tests.df11_cases import KINDS, compress_product, make_case, random_code_case
+from tests.df11_cases import KINDS, compress_product, make_case, random_code_case, short_positions_case
 
 pytestmark = pytest.mark.gpu
 
@@ -156,6 +156,39 @@ def test_gpu_reads_reference_encoder_streams(oracle):
     assert np.array_equal(gpu_decode(c), w)
 
 
+def test_gpu_reads_positions_one_entry_short(oracle):
+    """The reference encoder leaves output_positions one entry short when the last code
+    crosses a block boundary and ends on a byte boundary (dfloat11_utils.py:146-162):
+    n_blocks entries, the last being the element count.  The array goes to the device
+    exactly as the reference would have saved it, unpadded."""
+    print("case positions one short", flush=True)
+    from oracle.df11_oracle import EOF
+    table = {1: (8, 0b10000000), 2: (16, 0b0000000000000001), EOF: (16, 0)}
+    data = np.array([1] * 4095 + [2], np.uint8)
+    enc, gaps, pos = oracle.c_encode(data, table)
+    luts = np.zeros((3, 256), np.uint8)
+    luts[0, :] = 1
+    luts[0, 0] = 255
+    luts[1, :] = 2
+    luts[2, 1], luts[2, 2] = 8, 16
+    sm = (np.arange(data.size) % 251).astype(np.uint8)
+    assert pos.size == 2 and -(-enc.size // 4096) == 2 and int(pos[-1]) == data.size
+    c = dict(luts=luts, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps)
+    g = to_gpu(c)
+    assert g["output_positions"].numel() == 4 * 2          # n_blocks entries, not n_blocks + 1
+    D.validate_stream(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"])
+    want = oracle.merge_bf16(data, sm)
+    assert np.array_equal(gpu_decode(c), want)
+    # multi-block streams with realistic code lengths whose positions are one short
+    for seed, n_full in ((1, 1), (2, 3), (3, 9)):
+        print(f"case positions one short, {n_full + 1} blocks", flush=True)
+        w, c = short_positions_case(oracle, seed, n_full)
+        ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"], c["output_positions"], c["gaps"])
+        assert np.array_equal(ref, w)
+        got = gpu_decode(c)
+        assert np.array_equal(got, w)
+
+
 def test_gpu_does_not_write_outside_output():
     print("case guard bands", flush=True)
     w = make_case("normal", 77_777, 89)
@@ -251,13 +284,14 @@ def test_gpu_llama_block_round_trip():
     assert torch.equal(out.view(torch.int16), w.view(torch.int16))
 
 
-@pytest.mark.parametrize("kind", ["outliers", "uniform256", "zeros"])
-def test_gpu_embedding_sized_adversarial_round_trip(kind):
-    """151936 x 4096 (622 329 856 elements) with an adversarial exponent mix: encode ->
-    decode is the identity at the largest tensor size of the Qwen3-8B shape."""
-    print(f"case embedding {kind}", flush=True)
+@pytest.mark.parametrize("rows,cols", [(151936, 4096), (4096, 14336)])
+@pytest.mark.parametrize("kind", ["laplace", "outliers", "uniform256", "zeros"])
+def test_gpu_embedding_sized_adversarial_round_trip(kind, rows, cols):
+    """151936 x 4096 (622 329 856 elements, the largest tensor of the Qwen3-8B shape) and
+    4096 x 14336 with an adversarial exponent mix: encode -> decode is the identity."""
+    print(f"case {rows}x{cols} {kind}", flush=True)
     import bench_extra
-    w = bench_extra.make_mix(torch, kind, 151936 * 4096, torch.device(DEV), seed=23)
+    w = bench_extra.make_mix(torch, kind, rows * cols, torch.device(DEV), seed=23)
     from dfloat11_amd import dfloat11_utils as U
     w_cpu = w.cpu()
     _, counter = U.get_codec(w_cpu)

@@ -294,3 +294,23 @@ def test_decode_block_range(oracle):
         oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
                         c["output_positions"], c["gaps"], block_range=(b, b + 1), out=out)
     assert np.array_equal(out, w)
+
+
+def test_config_1_full_size_linear_through_the_cpu_path(oracle):
+    """BASELINE configuration 1 at its stated size: a 4096x4096 BF16 weight, N(0, 0.02)
+    from seed 0, compressed by the product encoder (8 bytes per thread, 512 threads per
+    block) and decoded by the CPU restatement of the reference kernel: bit-exact."""
+    import torch
+    from dfloat11_amd import dfloat11_utils as U
+    g = torch.Generator(device="cpu").manual_seed(0)
+    w = (torch.randn(4096, 4096, generator=g) * 0.02).to(torch.bfloat16).flatten()
+    codec, _ = U.get_codec(w)
+    luts = U.get_luts(codec.get_code_table())
+    enc, sm, pos, gaps, split = U.encode_weights([w], codec, 8, 512)
+    assert sm.numel() == 16_777_216 and split.numel() == 0
+    n_blocks = -(-enc.numel() // 4096)
+    assert 1300 < n_blocks < 1360 and pos.numel() == n_blocks + 1 and gaps.numel() == 320 * n_blocks
+    ratio = (enc.numel() + sm.numel() + gaps.numel() + 4 * pos.numel()) / (2 * sm.numel())
+    assert 0.66 < ratio < 0.69
+    got = oracle.c_decode(luts.numpy(), enc.numpy(), sm.numpy(), pos.numpy(), gaps.numpy())
+    assert np.array_equal(got, w.view(torch.int16).numpy().view(np.uint16))
