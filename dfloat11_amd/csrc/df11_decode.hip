@@ -25,6 +25,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/df11.h"
 #include "df11_core.h"
 
@@ -504,6 +506,97 @@ int groups_per_cu(size_t lds_bytes) {
   return n < 1 ? 1 : n;
 }
 
+// Enqueues the two load-time kernels that fill `ws` for one stream.
+int enqueue_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const uint32_t* output_positions,
+                    const uint8_t* gaps, int32_t n_luts, int64_t n_bytes, int64_t n_elements, uint8_t* ws,
+                    const DeviceInfo& info, hipStream_t s) {
+  const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  hipLaunchKernelGGL(build_tables_kernel, dim3(kTableEntries / 256), dim3(256), 0, s, luts, (int)n_luts,
+                     ws, (uint32_t)n_blocks);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e);
+  if (n_blocks > 0) {
+    IndexArgs a;
+    a.luts = luts;
+    a.codes = encoded_exponent;
+    a.positions = output_positions;
+    a.gaps = gaps;
+    a.ws = ws;
+    a.n_bytes = n_bytes;
+    a.n_elements = n_elements;
+    a.n_blocks = n_blocks;
+    a.n_luts = n_luts;
+    a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
+    const size_t lds_bytes = (size_t)kFixedLds + 64;
+    int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
+    if (grid > n_blocks) grid = n_blocks;
+    hipLaunchKernelGGL(index_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+  }
+  return DF11_OK;
+}
+
+// Enqueues the decode of one stream whose workspace `ws` is (or will be, in
+// stream order) filled.
+int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
+                   const uint8_t* gaps, uint16_t* outputs, int32_t n_luts, int64_t n_bytes,
+                   int64_t n_elements, const uint8_t* ws, int32_t max_elems_per_subblock,
+                   const DeviceInfo& info, hipStream_t s) {
+  if (max_elems_per_subblock <= 0 || max_elems_per_subblock > kMaxElemsPerSub)
+    max_elems_per_subblock = kMaxElemsPerSub;
+  DecodeSizes z;
+  z.n_bytes = n_bytes;
+  z.n_elements = n_elements;
+  z.n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  z.n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
+  z.n_luts = n_luts;
+  z.stage_cap = stage_capacity(max_elems_per_subblock);
+  z.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
+  z.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
+             (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
+
+  const size_t lds_bytes = (size_t)kFixedLds + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
+  int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
+  const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
+  if (grid > needed) grid = needed;
+
+  hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, luts,
+                     encoded_exponent, sign_mantissa, gaps, outputs, ws, z);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? DF11_OK : hip_fail(e);
+}
+
+// ---------------------------------------------------------------------------
+// Library-owned workspace for callers that cannot allocate device memory.
+// `scratch` is a host-side stand-in for the device array: host code never uses
+// the name as an address, only the per-device pointer that
+// hipGetSymbolAddress returns (each GPU holds its own copy of the array).
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) uint8_t scratch[DF11_STATIC_WORKSPACE_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint8_t* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+int scratch_of_current_device(uint8_t** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e);
+  if (dev < 0 || dev >= kMaxDevices) return DF11_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e);
+    if (!p) return DF11_ERR_HIP;
+    g_scratch_ptr[dev] = static_cast<uint8_t*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return DF11_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -516,7 +609,7 @@ const char* df11_error_string(int code) {
     case DF11_ERR_INVALID_ARGUMENT: return "invalid argument";
     case DF11_ERR_UNSUPPORTED: return "unsupported configuration";
     case DF11_ERR_HIP: return "HIP runtime error";
-    case DF11_ERR_CAPACITY: return "output buffer too small";
+    case DF11_ERR_CAPACITY: return "buffer too small or fixed capacity exceeded";
     case DF11_ERR_FORMAT: return "code not expressible in the DF11 LUT layout";
     default: return "unknown error";
   }
@@ -544,30 +637,10 @@ int df11_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const uin
   if (n_blocks >= ((int64_t)1 << 28)) return DF11_ERR_UNSUPPORTED;
   uint8_t* ws = static_cast<uint8_t*>(workspace);
 
-  hipLaunchKernelGGL(build_tables_kernel, dim3(kTableEntries / 256), dim3(256), 0, s, luts, (int)n_luts,
-                     ws, (uint32_t)n_blocks);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return hip_fail(e);
-
-  if (n_blocks > 0) {
-    IndexArgs a;
-    a.luts = luts;
-    a.codes = encoded_exponent;
-    a.positions = output_positions;
-    a.gaps = gaps;
-    a.ws = ws;
-    a.n_bytes = n_bytes;
-    a.n_elements = n_elements;
-    a.n_blocks = n_blocks;
-    a.n_luts = n_luts;
-    a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
-    const size_t lds_bytes = (size_t)kFixedLds + 64;
-    int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
-    if (grid > n_blocks) grid = n_blocks;
-    hipLaunchKernelGGL(index_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, a);
-    e = hipGetLastError();
-    if (e != hipSuccess) return hip_fail(e);
-  }
+  if (int rc = enqueue_prepare(luts, encoded_exponent, output_positions, gaps, n_luts, n_bytes, n_elements, ws,
+                               info, s))
+    return rc;
+  hipError_t e = hipSuccess;
   if (max_elems_per_subblock) {
     WorkspaceHeader h;
     e = hipMemcpyAsync(&h, ws, sizeof h, hipMemcpyDeviceToHost, s);
@@ -603,34 +676,41 @@ int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint
     return DF11_ERR_INVALID_ARGUMENT;
   if ((reinterpret_cast<uintptr_t>(workspace) & 15) || (reinterpret_cast<uintptr_t>(outputs) & 1))
     return DF11_ERR_INVALID_ARGUMENT;
-  if (max_elems_per_subblock <= 0 || max_elems_per_subblock > kMaxElemsPerSub)
-    max_elems_per_subblock = kMaxElemsPerSub;
-
+  if (n_elements >= ((int64_t)1 << 32)) return DF11_ERR_UNSUPPORTED;   // positions are u32
   DeviceInfo info;
   if (int rc = device_info(info)) return rc;
+  return enqueue_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements,
+                        static_cast<const uint8_t*>(workspace), max_elems_per_subblock, info,
+                        static_cast<hipStream_t>(stream));
+}
 
+int df11_decode_static_workspace(const uint8_t* luts, const uint8_t* encoded_exponent,
+                                 const uint8_t* sign_mantissa, const uint32_t* output_positions,
+                                 const uint8_t* gaps, uint16_t* outputs, int32_t n_luts, int64_t n_bytes,
+                                 int64_t n_elements, int32_t max_elems_per_subblock, void* stream) {
+  if (n_bytes < 0 || n_elements < 0 || n_luts < 2) return DF11_ERR_INVALID_ARGUMENT;
+  if (n_bytes == 0 || n_elements == 0) return DF11_OK;
+  if (!luts || !encoded_exponent || !sign_mantissa || !output_positions || !gaps || !outputs)
+    return DF11_ERR_INVALID_ARGUMENT;
+  if ((reinterpret_cast<uintptr_t>(output_positions) & 3) || (reinterpret_cast<uintptr_t>(outputs) & 1))
+    return DF11_ERR_INVALID_ARGUMENT;
   if (n_elements >= ((int64_t)1 << 32)) return DF11_ERR_UNSUPPORTED;   // positions are u32
-  DecodeSizes z;
-  z.n_bytes = n_bytes;
-  z.n_elements = n_elements;
-  z.n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
-  z.n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
-  z.n_luts = n_luts;
-  z.stage_cap = stage_capacity(max_elems_per_subblock);
-  z.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
-  z.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
-             (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
-
-  const size_t lds_bytes = (size_t)kFixedLds + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
-  int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
-  const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
-  if (grid > needed) grid = needed;
-
-  hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes,
-                     static_cast<hipStream_t>(stream), luts, encoded_exponent, sign_mantissa, gaps,
-                     outputs, static_cast<const uint8_t*>(workspace), z);
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? DF11_OK : hip_fail(e);
+  // the stream's workspace must fit the library's static array
+  if (n_bytes > (int64_t)DF11_STATIC_MAX_STREAM_BYTES) return DF11_ERR_CAPACITY;
+  const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
+  if (workspace_bytes(n_blocks) > (int64_t)DF11_STATIC_WORKSPACE_BYTES) return DF11_ERR_CAPACITY;
+  DeviceInfo info;
+  if (int rc = device_info(info)) return rc;
+  uint8_t* ws = nullptr;
+  if (int rc = scratch_of_current_device(&ws)) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // The header word that accumulates a maximum is reset by build_tables_kernel
+  // itself; tables and positions are overwritten in full for this stream's size.
+  if (int rc = enqueue_prepare(luts, encoded_exponent, output_positions, gaps, n_luts, n_bytes, n_elements, ws,
+                               info, s))
+    return rc;
+  return enqueue_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements, ws,
+                        max_elems_per_subblock, info, s);
 }
 
 }  // extern "C"

@@ -8,7 +8,8 @@
  * Conventions: every function returns DF11_OK (0) or a negative DF11_ERR_*
  * code; df11_error_string() names it.  The library never allocates or frees
  * device memory: kernels are enqueued on the caller's stream and the caller owns
- * every buffer until that work completes.  Only df11_prepare (load time) may
+ * every buffer until that work completes (df11_decode_static_workspace keeps its
+ * workspace in a fixed device array of the library instead).  Only df11_prepare (load time) may
  * wait for the stream; df11_decode never synchronises.
  * `stream` is a hipStream_t passed as void* (NULL = the default stream).
  */
@@ -26,7 +27,7 @@ extern "C" {
 #define DF11_ERR_INVALID_ARGUMENT (-1)
 #define DF11_ERR_UNSUPPORTED (-2)
 #define DF11_ERR_HIP (-3)           /* a HIP runtime call failed; see df11_last_hip_error() */
-#define DF11_ERR_CAPACITY (-4)      /* an output buffer is too small */
+#define DF11_ERR_CAPACITY (-4)      /* a buffer is too small, or the input exceeds a fixed capacity */
 #define DF11_ERR_FORMAT (-5)        /* the code cannot be expressed in the DF11 LUT layout */
 
 /* Format constants (reference: dfloat11/dfloat11.py:45-46). */
@@ -90,6 +91,33 @@ int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint
                 const uint32_t *output_positions, const uint8_t *gaps, uint16_t *outputs,
                 int32_t n_luts, int64_t n_bytes, int64_t n_elements,
                 const void *workspace, int32_t max_elems_per_subblock, void *stream);
+
+/*
+ * df11_prepare + df11_decode in one call, with the workspace in a device array
+ * that the library itself holds (DF11_STATIC_WORKSPACE_BYTES per GPU, resident
+ * from the first call on that GPU until the process ends).  No counterpart in
+ * the reference: it is for callers that cannot allocate device memory or wait
+ * for the device -- code under HIP graph capture, serving loops, harnesses that
+ * forbid hipMalloc.  The call allocates and frees nothing, never synchronises,
+ * and enqueues three kernels on `stream` (tables, sub-block positions, decode).
+ * Arguments as for df11_decode, without the workspace.
+ *   max_elems_per_subblock  an upper bound on the elements any 512-byte
+ *               sub-block produces, if the caller knows one (it sizes the LDS
+ *               staging; too small a bound truncates sub-blocks); <= 0 selects
+ *               the format's worst case (4096), which is always safe
+ * Streams of more than DF11_STATIC_MAX_STREAM_BYTES bytes of encoded_exponent
+ * are rejected with DF11_ERR_CAPACITY.  All calls on one GPU share the one
+ * array: calls that overlap in time on the same GPU (different streams) race;
+ * the caller serialises them.  The first call on a GPU looks the array's device
+ * address up (hipGetSymbolAddress); make that call outside a graph capture.
+ */
+#define DF11_STATIC_WORKSPACE_BYTES 4194304
+#define DF11_STATIC_MAX_STREAM_BYTES 534499328   /* 130493 bitstream blocks */
+int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exponent,
+                                 const uint8_t *sign_mantissa, const uint32_t *output_positions,
+                                 const uint8_t *gaps, uint16_t *outputs, int32_t n_luts,
+                                 int64_t n_bytes, int64_t n_elements,
+                                 int32_t max_elems_per_subblock, void *stream);
 
 /*
  * Streaming device copy of n_bytes (multiple of 16, both pointers 16-byte
