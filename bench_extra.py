@@ -25,11 +25,15 @@ if ROOT not in sys.path:
 from bench import HBM_PEAK_GBPS, algorithmic_bytes   # noqa: E402
 
 MIX_SHAPES = [("embedding", 151936, 4096), ("mlp_down", 4096, 14336)]
+ALL_SHAPES = MIX_SHAPES + [("attn_proj", 4096, 4096)]
+MIXES = ("laplace", "outliers", "uniform256", "zeros")
 
 
 def make_mix(torch, kind, n, device, seed):
     """BF16 tensor of n elements with the named exponent distribution."""
     g = torch.Generator(device=device).manual_seed(seed)
+    if kind == "normal":                       # N(0, 0.02), the usual weight initialisation
+        return (torch.randn(n, generator=g, device=device) * 0.02).to(torch.bfloat16)
     if kind == "laplace":                      # Laplace(0, 0.01)
         u = torch.rand(n, generator=g, device=device) - 0.5
         x = -0.01 * torch.sign(u) * torch.log1p(-2 * u.abs().clamp(max=0.49999997))
@@ -100,8 +104,8 @@ def time_decode(torch, w, steps, warmup):
 
 def run_mixes(a, torch, dev):
     ok = True
-    for kind in ("laplace", "outliers", "uniform256", "zeros"):
-        for name, rows, cols in MIX_SHAPES:
+    for kind in ([a.mix] if a.mix else MIXES):
+        for name, rows, cols in ([t for t in ALL_SHAPES if t[0] == a.tensor] if a.tensor else MIX_SHAPES):
             w = make_mix(torch, kind, rows * cols, dev, seed=7)
             r = time_decode(torch, w, a.steps, a.warmup)
             del w
@@ -324,6 +328,8 @@ def run_flux(a, torch, dev):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--workload", choices=["mixes", "flux-offload"], required=True)
+    ap.add_argument("--mix", choices=MIXES + ("normal",), default=None, help="mixes: only this distribution")
+    ap.add_argument("--tensor", choices=[t[0] for t in ALL_SHAPES], default=None, help="mixes: only this tensor")
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--double_blocks", type=int, default=19)

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kThreads) void index_kernel(const IndexArgs a) {
 
 // ---------------------------------------------------------------------------
 // Decode kernel.
-// LDS layout (dynamic): tables | byte LUT rows + length row | 8 staging areas
+// LDS layout (dynamic): tables | the byte LUT rows that exist + length row | 8 staging areas
 //
 // Everything that is the same for the 64 lanes of a wavefront (sub-block index,
 // output position, plan of the write-out) is kept wavefront-uniform on purpose,
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   const int n_rows = min(z.n_luts - 1, kMaxDecodeRows);
   uint8_t* lds_tables = lds;
   uint8_t* lds_rows = lds + kTablesBytes;
-  uint8_t* stage = lds_rows + (kMaxDecodeRows + 1) * 256 + wave * (uint32_t)z.stage_cap;
+  uint8_t* stage = lds_rows + (n_rows + 1) * 256 + wave * (uint32_t)z.stage_cap;
   const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
   // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
   // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
@@ -556,7 +556,10 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   z.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
              (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
 
-  const size_t lds_bytes = (size_t)kFixedLds + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
+  // LDS: tables, the byte LUT rows that exist plus the length row, one staging area per wavefront
+  const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
+  const size_t lds_bytes = (size_t)kTablesBytes + (size_t)(n_rows + 1) * 256 +
+                           (size_t)kWavesPerGroup * (size_t)z.stage_cap;
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;

@@ -20,6 +20,7 @@ What differs from the reference, by design:
 import json
 import os
 import re
+import weakref
 from sys import stderr
 from typing import Dict, Optional, Union
 
@@ -65,35 +66,37 @@ class TensorManager:
 
 class _OffloadPrefetcher:
     """Copies the offloaded streams of the NEXT compressed module to the device on
-    a side stream while the current one decodes and runs.  The order of modules is
-    learnt from the order in which their hooks fire; two device staging slots per
-    tensor name alternate, and events order copy -> decode -> slot reuse."""
+    a side stream while the current one decodes and runs.  Which module follows
+    which is learnt from the order in which their hooks fire; two device staging
+    slots per tensor name alternate, and events order copy -> decode -> slot reuse.
+
+    Modules are referenced weakly: a model that is deleted takes its pinned host
+    streams with it, and when the last offloaded module seen on a device is gone
+    the device's staging slots and side stream are released too."""
 
     def __init__(self):
-        self.order = []          # modules in execution order (learnt on the first pass)
-        self.index = {}          # id(module) -> position in order
+        self.successor = weakref.WeakKeyDictionary()   # module -> weakref of the module that ran after it
+        self.pending = weakref.WeakKeyDictionary()     # module -> (dict name -> device tensor, copy-done event, parity)
+        self.seen = weakref.WeakKeyDictionary()        # module -> device it was registered for
+        self.last = {}           # device -> (weakref of the module whose hook fired last, its parity)
+        self.live = {}           # device -> number of living modules registered for it
         self.streams = {}        # device -> side stream
         self.slots = {}          # (device, parity, name) -> device tensor
-        self.pending = {}        # id(module) -> (dict name -> device tensor, copy-done event)
         self.slot_free = {}      # (device, parity) -> event recorded after the last decode that read the slot
-        self.slot_owner = {}     # (device, parity) -> id(module) whose streams the slot holds or is receiving
+        self.slot_owner = {}     # (device, parity) -> weakref of the module whose streams the slot holds or is receiving
+        self.finalizers = weakref.WeakKeyDictionary()  # module -> the finalizer that reports its death
+        self.generation = getattr(self, 'generation', 0) + 1   # finalizers of an earlier reset() are void
         self.enabled = True
 
-    def _slot(self, device, parity, name, like):
-        key = (device, parity, name)
-        buf = self.slots.get(key)
-        if buf is None or buf.numel() < like.numel():
-            buf = torch.empty(like.numel(), dtype=like.dtype, device=device)
-            self.slots[key] = buf
-        return buf[:like.numel()]
-
-    def _issue(self, module, device):
-        """Start the host-to-device copies of `module`'s offloaded tensors on the side stream."""
-        pos = self.index[id(module)]
-        parity = pos & 1
+    # -- the three places that touch the GPU, kept apart so that the bookkeeping can be tested without one
+    def _side_stream(self, device):
         side = self.streams.get(device)
         if side is None:
             side = self.streams[device] = torch.cuda.Stream(device=device)
+        return side
+
+    def _copy_to_slots(self, module, device, parity):
+        side = self._side_stream(device)
         free = self.slot_free.get((device, parity))
         with torch.cuda.stream(side):
             if free is not None:
@@ -105,48 +108,98 @@ class _OffloadPrefetcher:
                 tensors[name] = dst
             done = torch.cuda.Event()
             done.record(side)
-        self.pending[id(module)] = (tensors, done, parity)
-        self.slot_owner[(device, parity)] = id(module)
+        return tensors, done
+
+    def _wait_and_mark(self, device, tensors, done):
+        current = torch.cuda.current_stream(device)
+        current.wait_event(done)
+        for t in tensors.values():
+            t.record_stream(current)          # allocated on the side stream, read on this one
+
+    def _decode_done_event(self, device):
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(device))
+        return ev
+
+    # -- bookkeeping
+    def _slot(self, device, parity, name, like):
+        key = (device, parity, name)
+        buf = self.slots.get(key)
+        if buf is None or buf.numel() < like.numel():
+            buf = torch.empty(like.numel(), dtype=like.dtype, device=device)
+            self.slots[key] = buf
+        return buf[:like.numel()]
+
+    def _register(self, module, device):
+        if self.seen.get(module) == device:
+            return
+        if module in self.seen:                # moved to another device: counted there from now on
+            self.finalizers.pop(module).detach()
+            self._released(self.seen[module], self.generation)
+        self.seen[module] = device
+        self.live[device] = self.live.get(device, 0) + 1
+        self.finalizers[module] = weakref.finalize(module, self._released, device, self.generation)
+
+    def _released(self, device, generation):
+        """A module registered for `device` is gone (or has moved away)."""
+        if generation != self.generation:
+            return
+        left = self.live.get(device, 0) - 1
+        if left > 0:
+            self.live[device] = left
+            return
+        self.live.pop(device, None)
+        self.streams.pop(device, None)
+        self.last.pop(device, None)
+        for table in (self.slots, self.slot_free, self.slot_owner):
+            for key in [k for k in table if k[0] == device]:
+                del table[key]
+
+    def _issue(self, module, device, parity):
+        """Start the host-to-device copies of `module`'s offloaded tensors on the side stream."""
+        tensors, done = self._copy_to_slots(module, device, parity)
+        self.pending[module] = (tensors, done, parity)
+        self.slot_owner[(device, parity)] = weakref.ref(module)
 
     def _prefetched(self, module, device):
         """True while the copies issued for `module` are still what its slot holds.
         When modules run in another order than the one learnt (a block skipped, a
         new one in between), a slot can be handed to another module before the
         one it was filled for ever runs."""
-        entry = self.pending.get(id(module))
+        entry = self.pending.get(module)
         if entry is None:
             return False
-        if self.slot_owner.get((device, entry[2])) != id(module):
-            del self.pending[id(module)]
+        owner = self.slot_owner.get((device, entry[2]))
+        if owner is None or owner() is not module:
+            del self.pending[module]
             return False
         return True
 
     def fetch(self, module, device):
         """Device copies of `module`'s offloaded tensors, ready on the current stream."""
-        key = id(module)
-        if key not in self.index:
-            self.index[key] = len(self.order)
-            self.order.append(module)
+        self._register(module, device)
+        last = self.last.get(device)
+        if last is not None:
+            before = last[0]()
+            if before is not None and before is not module:
+                self.successor[before] = weakref.ref(module)
         if not self._prefetched(module, device):
-            self._issue(module, device)       # first pass, or the prediction missed
-        tensors, done, parity = self.pending.pop(key)
-        current = torch.cuda.current_stream(device)
-        current.wait_event(done)
-        for t in tensors.values():
-            t.record_stream(current)          # allocated on the side stream, read on this one
+            # first pass, or the prediction missed: the slot the previous module is not using
+            self._issue(module, device, (last[1] ^ 1) if last is not None else 0)
+        tensors, done, parity = self.pending.pop(module)
+        self._wait_and_mark(device, tensors, done)
+        self.last[device] = (weakref.ref(module), parity)
         return tensors, parity
 
     def after_decode(self, module, device, parity):
         """Called once the decode of `module` is enqueued: frees its slot for reuse and
-        prefetches the module expected to run next."""
-        ev = torch.cuda.Event()
-        ev.record(torch.cuda.current_stream(device))
-        self.slot_free[(device, parity)] = ev
-        pos = self.index[id(module)]
-        if self.enabled and pos + 1 < len(self.order):   # successor known from an earlier pass
-            nxt = self.order[pos + 1]
-            if hasattr(nxt, 'offloaded_tensors') and not self._prefetched(nxt, device):
-                self._issue(nxt, device)
+        prefetches the module expected to run next into the other slot."""
+        self.slot_free[(device, parity)] = self._decode_done_event(device)
+        nxt = self.successor.get(module)
+        nxt = nxt() if nxt is not None else None
+        if self.enabled and nxt is not None and getattr(nxt, 'offloaded_tensors', None) \
+                and not self._prefetched(nxt, device):
+            self._issue(nxt, device, parity ^ 1)
 
     def reset(self):
         self.__init__()
@@ -155,20 +208,45 @@ class _OffloadPrefetcher:
 _prefetcher = _OffloadPrefetcher()
 
 
+_STREAM_NAMES = ('luts', 'encoded_exponent', 'sign_mantissa', 'output_positions', 'gaps')
+
+
+def _stream_state(module):
+    """The five stream tensors of a module as (object, in-place version) pairs: what the
+    cached launch arguments and the decode workspace were derived from.  A tensor that
+    was replaced shows as another object, one written in place (load_state_dict copies
+    into the existing buffers) as another version."""
+    state = []
+    for name in _STREAM_NAMES:
+        t = module._buffers.get(name)
+        if t is None and name in getattr(module, 'offloaded_tensors', {}):
+            t = module.offloaded_tensors[name]
+        state.append((t, t._version if t is not None else -1))
+    return tuple(state)
+
+
+def _same_streams(module, state):
+    now = _stream_state(module)
+    return all(a[0] is b[0] and a[1] == b[1] for a, b in zip(now, state))
+
+
 def _workspace_for(module, device, encoded_exponent, n_elements):
-    """The module's decode workspace on `device`, built on first use there."""
+    """The module's decode workspace on `device`: built on first use there, and again
+    when any of the stream tensors it was derived from has been replaced or rewritten."""
+    cached = module.__dict__.get('_df11_workspace_state')
     ws = getattr(module, '_df11_workspace', None)
-    if ws is None or ws.device != device:
-        if ws is None:   # first use: check the layout once, before anything is launched on it
-            sign_mantissa = (module.offloaded_tensors['sign_mantissa'] if hasattr(module, 'offloaded_tensors')
-                             else module.sign_mantissa)
-            _decode.validate_stream(module.luts, encoded_exponent, sign_mantissa, module.output_positions,
-                                    module.gaps, type(module).__name__)
+    if ws is None or ws.device != device or cached is None or not _same_streams(module, cached):
+        # check the layout before anything is launched on it
+        sign_mantissa = module.offloaded_tensors['sign_mantissa'] \
+            if 'sign_mantissa' in getattr(module, 'offloaded_tensors', {}) else module.sign_mantissa
+        _decode.validate_stream(module.luts, encoded_exponent, sign_mantissa, module.output_positions,
+                                module.gaps, type(module).__name__)
         ws, max_sub = _decode.prepare(module.luts, encoded_exponent, module.output_positions,
                                       module.gaps, n_elements)
         # plain attributes, not buffers: derived data must not leak into state_dict()
         object.__setattr__(module, '_df11_workspace', ws)
         object.__setattr__(module, '_df11_max_sub', max_sub)
+        object.__setattr__(module, '_df11_workspace_state', _stream_state(module))
     return module._df11_workspace, module._df11_max_sub
 
 
@@ -195,20 +273,20 @@ def get_hook(threads_per_block, bytes_per_thread):
         # later calls are one library call and nothing else.
         plan = module.__dict__.get('_df11_plan')
         if plan is not None and plan[0] is TensorManager._tensors.get(device) \
-                and plan[1] is module._buffers.get('encoded_exponent') \
-                and plan[2] is module._buffers.get('sign_mantissa') and plan[3] is module._buffers.get('luts') \
-                and all(owner.__dict__.get('weight') is view for owner, view in plan[5]):
-            _decode.launch(plan[4], device)
+                and _same_streams(module, plan[1]) \
+                and all(owner.__dict__.get('weight') is view for owner, view in plan[3]):
+            _decode.launch(plan[2], device)
             return
 
+        # Each of the two large streams comes from the prefetcher when the module holds it in
+        # host memory, else from the module's own buffer (a module may have only one of them
+        # offloaded: reference dfloat11.py:123-128 moves whatever offloaded_tensors holds).
         parity = None
-        if hasattr(module, 'offloaded_tensors'):
+        fetched = {}
+        if getattr(module, 'offloaded_tensors', None):
             fetched, parity = _prefetcher.fetch(module, device)
-            encoded_exponent = fetched['encoded_exponent']
-            sign_mantissa = fetched['sign_mantissa']
-        else:
-            encoded_exponent = module.encoded_exponent
-            sign_mantissa = module.sign_mantissa
+        encoded_exponent = fetched['encoded_exponent'] if 'encoded_exponent' in fetched else module.encoded_exponent
+        sign_mantissa = fetched['sign_mantissa'] if 'sign_mantissa' in fetched else module.sign_mantissa
 
         n_elements = sign_mantissa.numel()
         reconstructed = TensorManager.allocate_bfloat16(device, n_elements)
@@ -233,8 +311,8 @@ def get_hook(threads_per_block, bytes_per_thread):
         if parity is not None:
             _prefetcher.after_decode(module, device, parity)
         else:
-            object.__setattr__(module, '_df11_plan', (TensorManager._tensors.get(device), encoded_exponent,
-                                                      sign_mantissa, module.luts, bound, injected))
+            object.__setattr__(module, '_df11_plan', (TensorManager._tensors.get(device), _stream_state(module),
+                                                      bound, injected))
 
     return decode_hook
 

@@ -255,3 +255,116 @@ def test_compress_cli_on_a_local_checkpoint(tmp_path):
     want = torch.cat([base.get_submodule(f"model.layers.1.{n}").weight.detach().flatten()
                       for n in compress.LLM_PATTERNS[r"model\.layers\.\d+"]])
     assert layer["model.layers.1.sign_mantissa"].numel() == want.numel()
+
+
+class _StubPrefetcher(M._OffloadPrefetcher):
+    """The prefetcher's bookkeeping without a GPU: copies, waits and events are recorded, not run."""
+
+    def __init__(self):
+        super().__init__()
+        self.log = []
+
+    def _copy_to_slots(self, module, device, parity):
+        self.log.append(("copy", module.name, parity))
+        tensors = {name: self._slot(device, parity, name, host) for name, host in module.offloaded_tensors.items()}
+        for name, dst in tensors.items():
+            dst.copy_(module.offloaded_tensors[name])
+        return tensors, object()
+
+    def _wait_and_mark(self, device, tensors, done):
+        pass
+
+    def _decode_done_event(self, device):
+        return object()
+
+
+class _Offloaded(nn.Module):
+    def __init__(self, name, n):
+        super().__init__()
+        self.name = name
+        self.offloaded_tensors = {"encoded_exponent": torch.full((n,), len(name), dtype=torch.uint8),
+                                  "sign_mantissa": torch.arange(n, dtype=torch.uint8)}
+
+
+def test_prefetcher_learns_the_order_and_lets_go_of_dead_modules():
+    import gc
+    import weakref
+    p = _StubPrefetcher()
+    dev = torch.device("cpu")          # stands in for a GPU: the stub never touches it
+    mods = [_Offloaded(f"m{i}", 10 + i) for i in range(3)]
+
+    def forward(order):
+        for m in order:
+            tensors, parity = p.fetch(m, dev)
+            assert torch.equal(tensors["sign_mantissa"], m.offloaded_tensors["sign_mantissa"])
+            assert torch.equal(tensors["encoded_exponent"], m.offloaded_tensors["encoded_exponent"])
+            p.after_decode(m, dev, parity)
+
+    forward(mods)                      # first pass: every copy is issued by the module itself
+    assert [e[1] for e in p.log] == ["m0", "m1", "m2"]
+    assert [e[2] for e in p.log] == [0, 1, 0]          # the two slots alternate
+    p.log.clear()
+    forward(mods)                      # second pass: m0 copies itself, the others were copied one module ahead
+    assert [e[1] for e in p.log] == ["m0", "m1", "m2", "m0"]
+    p.log.clear()
+    forward([mods[0], mods[2]])        # a block skipped: the copy made for m1 is dropped, m2 fetches its own
+    assert [e[1] for e in p.log] == ["m1", "m2", "m0"] and not p._prefetched(mods[1], dev)
+    forward(mods)
+    # deleting the modules releases everything that was kept for them, without reset()
+    refs = [weakref.ref(m) for m in mods]
+    assert p.live == {dev: 3} and p.slots
+    del mods
+    gc.collect()
+    assert all(r() is None for r in refs)
+    assert not p.live and not p.slots and not p.slot_owner and not p.slot_free and not p.last
+    assert len(p.pending) == 0 and len(p.successor) == 0
+
+
+def test_prefetcher_reset_voids_earlier_finalizers():
+    import gc
+    p = _StubPrefetcher()
+    dev = torch.device("cpu")
+    old = _Offloaded("old", 4)
+    p.fetch(old, dev)
+    p.reset()
+    p.log = []
+    new = _Offloaded("new", 4)
+    tensors, parity = p.fetch(new, dev)
+    del old
+    gc.collect()
+    assert p.live == {dev: 1} and p.slots      # the death of a module from before the reset changes nothing
+
+
+def test_hook_takes_each_stream_from_where_it_is(monkeypatch):
+    """A module with only one of its two large streams offloaded (tensor names of different
+    modules interleave in a file and cpu_offload_blocks runs out in between): the hook
+    takes that stream from the prefetcher and the other from the module's buffer."""
+    calls = {}
+    mod = nn.Linear(4, 2, bias=False).to(torch.bfloat16)
+    delattr(mod, "weight")
+    mod.register_buffer("luts", torch.zeros(2, 256, dtype=torch.uint8))
+    mod.register_buffer("sign_mantissa", torch.arange(8, dtype=torch.uint8))
+    mod.register_buffer("output_positions", torch.zeros(8, dtype=torch.uint8))
+    mod.register_buffer("gaps", torch.zeros(320, dtype=torch.uint8))
+    mod.offloaded_tensors = {"encoded_exponent": torch.ones(16, dtype=torch.uint8)}
+    mod.split_positions = []
+    staged = torch.full((16,), 7, dtype=torch.uint8)
+
+    class FakeDevice:
+        type = "cuda"
+    monkeypatch.setattr(type(mod.luts), "device", property(lambda self: FakeDevice()), raising=False)
+    monkeypatch.setattr(M._prefetcher, "fetch", lambda module, device: ({"encoded_exponent": staged}, 1))
+    monkeypatch.setattr(M._prefetcher, "after_decode", lambda module, device, parity: calls.setdefault("after", parity))
+    monkeypatch.setattr(M.TensorManager, "allocate_bfloat16",
+                        staticmethod(lambda device, n: torch.zeros(n, dtype=torch.bfloat16)))
+    monkeypatch.setattr(M._decode, "validate_stream", lambda *a, **k: None)
+    monkeypatch.setattr(M._decode, "prepare", lambda *a, **k: (torch.zeros(16, dtype=torch.uint8), 5))
+
+    def bind(luts, enc, sm, pos, gaps, out, ws, max_sub):
+        calls["bind"] = (enc, sm)
+        return ()
+    monkeypatch.setattr(M._decode, "bind", bind)
+    monkeypatch.setattr(M._decode, "launch", lambda bound, device: calls.setdefault("launched", True))
+    M.get_hook((512,), 8)(mod, None)
+    assert calls["bind"][0] is staged and calls["bind"][1] is mod.sign_mantissa
+    assert calls["launched"] and calls["after"] == 1 and mod.weight.shape == (2, 4)

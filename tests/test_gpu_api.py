@@ -259,3 +259,60 @@ def test_flux_shaped_offloaded_pass_is_bit_identical():
     M._prefetcher.reset()
     M.TensorManager.clear()
     torch.cuda.empty_cache()
+
+
+def test_offloaded_model_is_collected_without_reset(tmp_path):
+    """An offloaded model that is deleted takes its pinned host streams with it, and the
+    prefetcher lets go of the device staging slots it kept for it (no manual reset())."""
+    print("case api offload, model deleted", flush=True)
+    import gc
+    import weakref
+    compress_model(make_model(8), PATTERNS, str(tmp_path), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path), device=DEV, bfloat16_model=make_model(9), cpu_offload=True)
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+    want = _reference_logits(8, ids)
+    with torch.no_grad():
+        for _ in range(3):
+            assert torch.equal(model(ids), want)
+    dev = torch.device(DEV)
+    assert M._prefetcher.live.get(dev) == 5 and any(k[0] == dev for k in M._prefetcher.slots)
+    layer = weakref.ref(model.layers[1])
+    host = weakref.ref(model.layers[1].offloaded_tensors["encoded_exponent"])
+    torch.cuda.synchronize()
+    del model
+    gc.collect()
+    assert layer() is None and host() is None
+    assert dev not in M._prefetcher.live and not any(k[0] == dev for k in M._prefetcher.slots)
+    assert len(M._prefetcher.pending) == 0 and len(M._prefetcher.successor) == 0
+
+
+def test_streams_rewritten_in_place_are_decoded_anew(tmp_path):
+    """load_state_dict copies a second model's streams into the existing buffers: the
+    objects stay, their contents change.  The launch arguments and the decode workspace
+    derived from the old contents must not be used again."""
+    print("case api streams rewritten in place", flush=True)
+    from safetensors.torch import load_file
+    M._prefetcher.reset()
+    a, b = make_model(10), make_model(10)
+    with torch.no_grad():
+        for p in b.parameters():          # the same values in another order: same code, same stream sizes
+            if p.dim() > 1:
+                p.copy_(p.flatten().flip(0).view_as(p))
+    ref_b = make_model(10)
+    ref_b.load_state_dict(b.state_dict())
+    compress_model(a, PATTERNS, str(tmp_path / "a"), check_correctness=False)
+    compress_model(b, PATTERNS, str(tmp_path / "b"), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path / "a"), device=DEV, bfloat16_model=make_model(9))
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+    with torch.no_grad():
+        assert torch.equal(model(ids), _reference_logits(10, ids))
+        assert torch.equal(model(ids), _reference_logits(10, ids))      # launch arguments bound by now
+        state_b = {k: v for k, v in load_file(str(tmp_path / "b" / "model.safetensors")).items()
+                   if not k.endswith("split_positions")}
+        before = model.layers[0].encoded_exponent
+        assert state_b["layers.0.encoded_exponent"].shape == before.shape
+        model.load_state_dict(state_b, strict=False)
+        assert model.layers[0].encoded_exponent is before               # rewritten in place
+        want = ref_b.to(DEV)(ids)
+        assert torch.equal(model(ids), want)
+        assert torch.equal(model(ids), want)
