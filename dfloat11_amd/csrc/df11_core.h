@@ -29,35 +29,70 @@ constexpr int kTableEntries = 1 << kK;
 //                      11-bit window, first code in byte 0;
 //                      word 1 ("meta"): bits consumed in byte 0, code count in
 //                      byte 1; 0 = the first code is longer than 11 bits
+//                      when the first code is longer than 11 bits, word 0 holds the
+//                      fused entry (below) of the root row for the window's first byte
 //   cntt u8[2048]      index (1<<r)|v, v = the next r bits (r < 11): how many codes
 //                      start inside those r bits
+//   rows u16[n_rows][256]  the byte LUT rows fused with the length row: bits 0-7 the
+//                      row's byte d, bits 8-14 the recorded code length of symbol d
+//                      (1 where it is 0), bit 15 set if d names a row that exists
+//                      (d >= 240 and 256 - d < n_rows): a pointer on levels 0-2
 constexpr int kDecOffset = 0;
 constexpr int kCntTailOffset = kTableEntries * 8;
-constexpr int kTablesBytes = kCntTailOffset + kTableEntries;
+constexpr int kRowsOffset = kCntTailOffset + kTableEntries;
 
 // Byte LUT rows a pointer entry can name: values 255..240 name rows 1..16.
 constexpr int kMaxDecodeRows = 17;
+constexpr int kRowBytes = 256 * 2;
+constexpr int kTablesBytes = kRowsOffset + kMaxDecodeRows * kRowBytes;   // the blob with every row present
+// Bytes of the blob a decode needs when the stream has n_rows decode rows.
+DF11_HD int tables_bytes(int n_rows) { return kRowsOffset + n_rows * kRowBytes; }
 
 struct Luts {
   const uint8_t* rows;   // n_rows decode rows of 256 bytes, then the length row
   int n_rows;            // decode rows present (root included), <= kMaxDecodeRows
 };
 
-// Hierarchical lookup of the code at the top of `window`.  A value >= 240 on
-// the first three levels names row 256 - value when that row exists.  A symbol
-// whose recorded length is 0 can only be reached through padding bits; it is
-// given length 1 so that every caller makes progress.
-DF11_HD void walk(const Luts& l, uint64_t window, uint32_t& sym, uint32_t& len) {
-  uint32_t d = l.rows[window >> 56];
+// Fused entry of byte `byte` of row `row`: what a hierarchical lookup needs to know
+// about that slot, in one 16-bit read.  A symbol whose recorded length is 0 can
+// only be reached through padding bits; it is given length 1 so that every
+// caller makes progress.
+constexpr uint32_t kRowPointer = 0x8000u;
+DF11_HD uint16_t make_row_entry(const Luts& l, uint32_t row, uint32_t byte) {
+  const uint32_t d = l.rows[row * 256u + byte];
+  uint32_t n = l.rows[(uint32_t)l.n_rows * 256u + d];
+  if (n > 127u) n = 127u;                      // a valid length is at most 32; keeps bit 15 for the flag
+  const bool names_row = d >= 240u && 256u - d < (uint32_t)l.n_rows;
+  return (uint16_t)(d | ((n ? n : 1u) << 8) | (names_row ? kRowPointer : 0u));
+}
+
+// The fused rows as the decode reads them (LDS on the device).
+struct Rows {
+  const uint8_t* e;   // u16[n_rows][256], 2-byte aligned
+};
+
+DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte) {
+  uint16_t v;
+  __builtin_memcpy(&v, static_cast<const uint8_t*>(__builtin_assume_aligned(r.e, 2)) + (row * 256u + byte) * 2u, 2);
+  return v;
+}
+
+// Hierarchical lookup of the code whose first 32 bits are `top` (first bit in
+// bit 31), continued from the root row's entry `e` for the first byte.  A value
+// >= 240 on the first three levels names row 256 - value when that row exists;
+// on the fourth level it is a symbol.
+DF11_HD void walk_from(const Rows& r, uint32_t e, uint32_t top, uint32_t& sym, uint32_t& len) {
 #pragma unroll
   for (int level = 1; level <= 3; ++level) {
-    const uint32_t row = 256u - d;
-    if (d < 240u || row >= (uint32_t)l.n_rows) break;
-    d = l.rows[row * 256u + (uint32_t)((window >> (56 - 8 * level)) & 0xffu)];
+    if (!(e & kRowPointer)) break;
+    e = row_entry(r, 256u - (e & 0xffu), (top >> (24 - 8 * level)) & 0xffu);
   }
-  sym = d;
-  const uint32_t n = l.rows[(uint32_t)l.n_rows * 256u + d];
-  len = n ? n : 1u;
+  sym = e & 0xffu;
+  len = (e >> 8) & 0x7fu;
+}
+
+DF11_HD void walk(const Rows& r, uint32_t top, uint32_t& sym, uint32_t& len) {
+  walk_from(r, row_entry(r, 0u, top >> 24), top, sym, len);
 }
 
 // ---- table construction (one entry per call) --------------------------------
@@ -118,7 +153,7 @@ DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_
     ++k;
   }
   meta = k ? (pos | (k << 8)) : 0u;
-  if (!k) syms = 0;
+  if (!k) syms = make_row_entry(l, 0u, idx >> (kK - 8));   // where the hierarchical lookup starts
 }
 
 DF11_HD uint8_t make_cnt_tail_entry(const Luts& l, uint32_t idx) {
@@ -184,6 +219,14 @@ DF11_HD uint64_t with_next(uint64_t w, uint32_t next, uint32_t c) {
   return w | (c >= 32u ? (uint64_t)next << (c - 32u) : (uint64_t)next >> (32u - c));
 }
 
+// The next 32 stream bits at the top of window `w`, of which the 64 - c topmost
+// bits are valid chunk bits and the rest zero (c < 64); `next` holds the 32 bits
+// that follow the chunk.
+DF11_HD uint32_t top_bits(uint64_t w, uint32_t next, uint32_t c) {
+  const uint32_t hi = (uint32_t)(w >> 32);
+  return c > 32u ? hi | (next >> (64u - c)) : hi;
+}
+
 // Byte offset of the table entry for the top kK bits of the window.
 DF11_HD uint32_t dec_offset(uint64_t w) { return ((uint32_t)(w >> 32) >> (32 - kK - 3)) & (uint32_t)((kTableEntries - 1) * 8); }
 
@@ -192,7 +235,7 @@ DF11_HD uint32_t dec_offset(uint64_t w) { return ((uint32_t)(w >> 32) >> (32 - k
 // Lookups stay inside the chunk (c <= 64 - kK), so the look-ahead is only needed
 // for codes longer than the table width; the last few bits are settled by one
 // lookup in the tail table.
-DF11_HD uint32_t count_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo,
+DF11_HD uint32_t count_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
                              uint32_t next, uint32_t gap) {
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   uint32_t cn = gap;                    // byte 0: bits consumed; bits 8 and up: codes counted
@@ -200,7 +243,7 @@ DF11_HD uint32_t count_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32
     uint32_t meta = load_as<uint32_t>(t.dec + dec_offset(w) + 4u);
     if (meta == 0u) {
       uint32_t s, n;
-      walk(l, with_next(w, next, cn & 0xffu), s, n);
+      walk(l, top_bits(w, next, cn & 0xffu), s, n);
       meta = n | 0x100u;
       DF11_KEEP_BRANCH();
     }
@@ -219,7 +262,7 @@ DF11_HD uint32_t count_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32
 // resolved are overwritten by the next store.  The last one to three symbols
 // are gathered in a register and stored exactly, so nothing is ever written at
 // or beyond p + remaining.
-DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo, uint32_t next,
+DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo, uint32_t next,
                         uint32_t gap, uint32_t remaining, uint8_t* p) {
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   uint32_t c = gap;                     // bit 7 is set once the look-ahead has been appended
@@ -234,7 +277,7 @@ DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo
     uint32_t syms = e.x, meta = e.y;
     if (meta == 0u) {
       uint32_t n;
-      walk(l, w, syms, n);              // at least 32 valid bits: c < 32, or already appended
+      walk_from(l, syms, (uint32_t)(w >> 32), syms, n);   // at least 32 valid bits: c < 32, or already appended
       meta = n | 0x100u;
       DF11_KEEP_BRANCH();
     }
@@ -256,7 +299,7 @@ DF11_HD void emit_chunk(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo
       uint32_t syms = e.x, meta = e.y;
       if (meta == 0u) {
         uint32_t n;
-        walk(l, w, syms, n);
+        walk_from(l, syms, (uint32_t)(w >> 32), syms, n);
         meta = n | 0x100u;
       }
       acc |= syms << got;
@@ -290,7 +333,7 @@ struct ChunkSyms {
   bool overflow;           // ran out of slots: count and syms are incomplete
 };
 
-DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Luts& l, uint32_t hi, uint32_t lo,
+DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
                                     uint32_t next, uint32_t gap) {
   ChunkSyms r;
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
@@ -303,7 +346,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Luts& l, uint32_t hi,
       uint32_t syms = e.x, meta = e.y;
       if (meta == 0u) {
         uint32_t len;
-        walk(l, with_next(w, next, c), syms, len);
+        walk_from(l, syms, top_bits(w, next, c), syms, len);
         meta = len | 0x100u;
         DF11_KEEP_BRANCH();
       }
@@ -329,7 +372,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Luts& l, uint32_t hi,
       uint32_t syms = e.x, meta = e.y;
       if (meta == 0u) {
         uint32_t len;
-        walk(l, w, syms, len);
+        walk_from(l, syms, (uint32_t)(w >> 32), syms, len);
         meta = len | 0x100u;
       }
       r.syms[kMainSlots + i] = syms;

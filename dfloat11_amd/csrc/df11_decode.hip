@@ -94,6 +94,9 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const uint8_t* __rest
   uint8_t* tables = ws + kWsTablesOffset;
   reinterpret_cast<uint2*>(tables + kDecOffset)[idx] = make_uint2(syms, meta);
   tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
+  uint16_t* fused = reinterpret_cast<uint16_t*>(tables + kRowsOffset);
+  for (uint32_t i = idx; i < (uint32_t)n_rows * 256u; i += (uint32_t)kTableEntries)
+    fused[i] = make_row_entry(l, i >> 8, i & 0xffu);
   if (idx < sizeof(WorkspaceHeader) / 4) {
     uint32_t v = 0;
     if (idx == 0) v = kWorkspaceMagic;
@@ -125,17 +128,15 @@ __global__ __launch_bounds__(kThreads) void index_kernel(const IndexArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_rows = min(a.n_luts - 1, kMaxDecodeRows);
   uint8_t* lds_tables = lds;
-  uint8_t* lds_rows = lds + kTablesBytes;
-  uint32_t* wave_sums = reinterpret_cast<uint32_t*>(lds_rows + (kMaxDecodeRows + 1) * 256);
+  uint32_t* wave_sums = reinterpret_cast<uint32_t*>(lds + kTablesBytes);
   {
     const uint4* src = reinterpret_cast<const uint4*>(a.ws + kWsTablesOffset);
     uint4* dst = reinterpret_cast<uint4*>(lds_tables);
-    for (int i = tid; i < kTablesBytes / 16; i += kThreads) dst[i] = src[i];
-    stage_rows(a.luts, a.n_luts, n_rows, lds_rows, tid, kThreads);
+    for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) dst[i] = src[i];
   }
   __syncthreads();
   const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
-  const Luts l{lds_rows, n_rows};
+  const Rows l{lds_tables + kRowsOffset};
   const int64_t n_gap_bytes = a.n_blocks * kGapBytesPerBlock;
   uint32_t* subpos = reinterpret_cast<uint32_t*>(a.ws + kWsSubposOffset);
   uint32_t my_max = 0;
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void index_kernel(const IndexArgs a) {
 
 // ---------------------------------------------------------------------------
 // Decode kernel.
-// LDS layout (dynamic): tables | the byte LUT rows that exist + length row | 8 staging areas
+// LDS layout (dynamic): tables | the fused LUT rows that exist | 8 staging areas
 //
 // Everything that is the same for the 64 lanes of a wavefront (sub-block index,
 // output position, plan of the write-out) is kept wavefront-uniform on purpose,
@@ -288,8 +289,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   const uint32_t wave = uniform(tid >> 6);
   const int n_rows = min(z.n_luts - 1, kMaxDecodeRows);
   uint8_t* lds_tables = lds;
-  uint8_t* lds_rows = lds + kTablesBytes;
-  uint8_t* stage = lds_rows + (n_rows + 1) * 256 + wave * (uint32_t)z.stage_cap;
+  uint8_t* stage = lds + tables_bytes(n_rows) + wave * (uint32_t)z.stage_cap;
   const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
   // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
   // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
@@ -306,8 +306,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   {
     const uint4* src = reinterpret_cast<const uint4*>(ws + kWsTablesOffset);
     uint4* dst = reinterpret_cast<uint4*>(lds_tables);
-    for (int i = tid; i < kTablesBytes / 16; i += kThreads) dst[i] = src[i];
-    stage_rows(luts, z.n_luts, n_rows, lds_rows, tid, kThreads);
+    for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) dst[i] = src[i];
   }
   // Replayed symbols are ORed into the staging area, which therefore starts out
   // zero and is cleared again after every sub-block.
@@ -315,7 +314,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   __syncthreads();   // the only workgroup barrier: tables are read-only from here on
 
   const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
-  const Luts l{lds_rows, n_rows};
+  const Rows l{lds_tables + kRowsOffset};
   const bool vec_ok = z.vec_ok != 0;
   const int64_t stride = (int64_t)gridDim.x * kWavesPerGroup;
   if (sub >= z.n_subs) return;
@@ -493,7 +492,6 @@ int device_info(DeviceInfo& info) {
   return DF11_OK;
 }
 
-constexpr int kFixedLds = kTablesBytes + (kMaxDecodeRows + 1) * 256;
 constexpr int kLdsPerCu = 160 * 1024;
 
 // Workgroups resident per CU.  Three (six wavefronts per SIMD) hide the decode
@@ -527,7 +525,7 @@ int enqueue_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const 
     a.n_blocks = n_blocks;
     a.n_luts = n_luts;
     a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
-    const size_t lds_bytes = (size_t)kFixedLds + 64;
+    const size_t lds_bytes = (size_t)kTablesBytes + 64;
     int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
     if (grid > n_blocks) grid = n_blocks;
     hipLaunchKernelGGL(index_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, a);
@@ -556,10 +554,9 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   z.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
              (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
 
-  // LDS: tables, the byte LUT rows that exist plus the length row, one staging area per wavefront
+  // LDS: tables, the fused LUT rows that exist, one staging area per wavefront
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
-  const size_t lds_bytes = (size_t)kTablesBytes + (size_t)(n_rows + 1) * 256 +
-                           (size_t)kWavesPerGroup * (size_t)z.stage_cap;
+  const size_t lds_bytes = (size_t)tables_bytes(n_rows) + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;

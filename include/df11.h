@@ -112,7 +112,7 @@ int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint
  * address up (hipGetSymbolAddress); make that call outside a graph capture.
  */
 #define DF11_STATIC_WORKSPACE_BYTES 4194304
-#define DF11_STATIC_MAX_STREAM_BYTES 534499328   /* 130493 bitstream blocks */
+#define DF11_STATIC_MAX_STREAM_BYTES 533385216   /* 130221 bitstream blocks */
 int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exponent,
                                  const uint8_t *sign_mantissa, const uint32_t *output_positions,
                                  const uint8_t *gaps, uint16_t *outputs, int32_t n_luts,

@@ -37,6 +37,10 @@ extern "C" int df11_emul_tables(const uint8_t* luts, int n_luts, uint8_t* tables
     memcpy(tables + kDecOffset + 8 * idx, e, 8);
     tables[kCntTailOffset + idx] = make_cnt_tail_entry(l, idx);
   }
+  for (uint32_t i = 0; i < (uint32_t)n_rows * 256u; ++i) {
+    const uint16_t e = make_row_entry(l, i >> 8, i & 0xffu);
+    memcpy(tables + kRowsOffset + 2 * i, &e, 2);
+  }
   return 0;
 }
 
@@ -50,11 +54,11 @@ extern "C" int df11_emul_prepare(const uint8_t* luts, const uint8_t* codes, cons
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
   memset(ws, 0, (size_t)workspace_bytes(n_blocks));
   df11_emul_tables(luts, n_luts, ws + kWsTablesOffset);
-  std::vector<uint8_t> rows((size_t)(n_rows + 1) * 256);
-  memcpy(rows.data(), luts, (size_t)n_rows * 256);
-  memcpy(rows.data() + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
-  const Tables t{ws + kWsTablesOffset + kDecOffset, ws + kWsTablesOffset + kCntTailOffset};
-  const Luts l{rows.data(), n_rows};
+  // the passes read an exact-size copy of the part of the blob a decode loads
+  Exact<uint8_t> blob((size_t)tables_bytes(n_rows));
+  memcpy(blob.p, ws + kWsTablesOffset, (size_t)tables_bytes(n_rows));
+  const Tables t{blob.p + kDecOffset, blob.p + kCntTailOffset};
+  const Rows l{blob.p + kRowsOffset};
   std::vector<uint32_t> subpos((size_t)n_blocks * kSubsPerBlock + 1);
   uint32_t max_sub = 0;
   for (int64_t blk = 0; blk < n_blocks; ++blk) {
@@ -113,14 +117,13 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   memset(c_out.p, 0xEE, ((size_t)n_elements + out_misalign) * 2);
   Exact<uint8_t> ws((size_t)workspace_bytes(n_blocks));
   df11_emul_prepare(luts, codes_p, c_pos.p, c_gaps.p, n_luts, n_bytes, n_elements, ws.p);
-  Exact<uint8_t> rows((size_t)(n_rows + 1) * 256);
-  memcpy(rows.p, luts, (size_t)n_rows * 256);
-  memcpy(rows.p + (size_t)n_rows * 256, luts + (size_t)(n_luts - 1) * 256, 256);
+  Exact<uint8_t> blob((size_t)tables_bytes(n_rows));   // what a workgroup copies into LDS
+  memcpy(blob.p, ws.p + kWsTablesOffset, (size_t)tables_bytes(n_rows));
   Exact<uint8_t> stage((size_t)stage_cap);
   memset(stage.p, 0, (size_t)stage_cap);   // the kernel clears each wavefront's area once at start
 
-  const Tables t{ws.p + kWsTablesOffset + kDecOffset, ws.p + kWsTablesOffset + kCntTailOffset};
-  const Luts l{rows.p, n_rows};
+  const Tables t{blob.p + kDecOffset, blob.p + kCntTailOffset};
+  const Rows l{blob.p + kRowsOffset};
   const uint32_t* subpos = reinterpret_cast<const uint32_t*>(ws.p + kWsSubposOffset);
   const bool codes_aligned = (reinterpret_cast<uintptr_t>(codes_p) & 7) == 0;
   const bool vec_ok = (reinterpret_cast<uintptr_t>(sm_p) & 7) == 0 &&

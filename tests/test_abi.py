@@ -27,9 +27,12 @@ def test_version_and_error_strings():
     assert hip.df11_version() == 2
     assert hip.df11_error_string(0) == b"ok"
     assert hip.df11_error_string(-1) == b"invalid argument"
-    # header + tables + (8 sub-blocks per 4096-byte block + 1) positions, rounded to 16
-    assert hip.df11_workspace_bytes(0) == 64 + 2048 * 8 + 2048 + 16
-    assert hip.df11_workspace_bytes(4097) == 64 + 2048 * 8 + 2048 + ((4 * 17 + 15) // 16) * 16
+    # header + tables + 17 fused LUT rows + (8 sub-blocks per 4096-byte block + 1) positions, rounded to 16
+    fixed = 64 + 2048 * 8 + 2048 + 17 * 512
+    assert hip.df11_workspace_bytes(0) == fixed + 16
+    assert hip.df11_workspace_bytes(4097) == fixed + ((4 * 17 + 15) // 16) * 16
+    # the largest stream whose workspace fits the library's static array, and the next larger one
+    assert hip.df11_workspace_bytes(533385216) <= 4194304 < hip.df11_workspace_bytes(533385216 + 4096)
 
 
 def test_argument_validation_needs_no_gpu():

@@ -192,10 +192,35 @@ def test_emulated_kernel_malformed_streams_stay_in_bounds(emul, tmp_path):
 def _host_tables(luts):
     L = ctypes.CDLL(os.path.join(EMUL_DIR, "libdf11_emul.so"))
     luts = np.ascontiguousarray(luts)
-    blob = np.zeros(2048 * 8 + 2048, np.uint8)
+    blob = np.zeros(2048 * 8 + 2048 + 17 * 512, np.uint8)      # dec | cntt | fused rows
     L.df11_emul_tables(_p(luts), luts.shape[0], _p(blob))
     dec = blob[: 2048 * 8].view(np.uint32).reshape(2048, 2)
-    return dec, blob[2048 * 8:]
+    return dec, blob[2048 * 8: 2048 * 8 + 2048]
+
+
+def _host_fused_rows(luts):
+    L = ctypes.CDLL(os.path.join(EMUL_DIR, "libdf11_emul.so"))
+    luts = np.ascontiguousarray(luts)
+    blob = np.zeros(2048 * 8 + 2048 + 17 * 512, np.uint8)
+    L.df11_emul_tables(_p(luts), luts.shape[0], _p(blob))
+    return blob[2048 * 8 + 2048:].view(np.uint16).reshape(17, 256)[: luts.shape[0] - 1]
+
+
+def _check_fused_rows(luts):
+    """The 16-bit rows the hierarchical lookup reads, from their definition: the LUT
+    byte, the recorded length of that byte taken as a symbol (1 where 0), and the flag
+    'names a row that exists'; an unresolved 11-bit pattern's table entry carries the
+    root row's fused entry for its first byte."""
+    luts = np.asarray(luts)
+    n_rows = luts.shape[0] - 1
+    d = luts[:n_rows].astype(np.uint32)
+    length = np.maximum(luts[-1].astype(np.uint32)[d], 1)
+    flag = (d >= 240) & (256 - d < n_rows)
+    want = (d | (length << 8) | (flag.astype(np.uint32) << 15)).astype(np.uint16)
+    assert np.array_equal(_host_fused_rows(luts), want)
+    dec, _ = _host_tables(luts)
+    unresolved = np.nonzero(dec[:, 1] == 0)[0]
+    assert np.array_equal(dec[unresolved, 0], want[0][unresolved >> 3].astype(np.uint32))
 
 
 def _first_code(bits, codes):
@@ -264,6 +289,7 @@ def _check_tables_against_code(codec, luts):
 def test_derived_tables_brute_force(emul, kind, n, seed):
     c = compress_product(make_case(kind, n, seed))
     _check_tables_against_code(c["codec"], c["luts"])
+    _check_fused_rows(c["luts"])
 
 
 @pytest.mark.parametrize("seed", [900, 905, 911, 922, 1059, 1065, 1165, 1195])
@@ -278,6 +304,7 @@ def test_derived_tables_brute_force_random_codes(emul, seed):
     _, cases = made
     for policy, c in cases.items():
         _check_tables_against_code(c["codec"], c["luts"])
+        _check_fused_rows(c["luts"])
 
 
 @pytest.mark.parametrize("chunk", range(8))

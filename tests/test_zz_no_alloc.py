@@ -75,7 +75,7 @@ def test_static_workspace_rejects_streams_beyond_its_capacity():
     lib = _native.hip_lib()
     one = torch.zeros(4096, dtype=torch.uint8, device=DEV)
     p = one.data_ptr()
-    too_many = 534499328 + 1        # DF11_STATIC_MAX_STREAM_BYTES + 1: only sizes are looked at before the refusal
+    too_many = 533385216 + 1        # DF11_STATIC_MAX_STREAM_BYTES + 1: only sizes are looked at before the refusal
     rc = lib.df11_decode_static_workspace(p, p, p, p, p, p, 2, too_many, 10, 0, None)
     assert rc == -4
     assert lib.df11_error_string(rc) == b"buffer too small or fixed capacity exceeded"
