@@ -11,7 +11,19 @@
 #define DF11_HD inline
 #endif
 
+// Pointers into workgroup memory (LDS) carry their address space on the device,
+// so that accesses compile to LDS instructions with constant parts of the address
+// in the instruction's offset field; on the host they are plain pointers.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define DF11_LDS __attribute__((address_space(3)))
+#else
+#define DF11_LDS
+#endif
+
 namespace df11 {
+
+typedef DF11_LDS uint8_t* LdsBytes;
+typedef const DF11_LDS uint8_t* ConstLdsBytes;
 
 constexpr int kChunkBytes = 8;        // bytes of bitstream owned by one thread
 constexpr int kThreads = 512;         // threads (chunks) per bitstream block
@@ -68,14 +80,10 @@ DF11_HD uint16_t make_row_entry(const Luts& l, uint32_t row, uint32_t byte) {
 
 // The fused rows as the decode reads them (LDS on the device).
 struct Rows {
-  const uint8_t* e;   // u16[n_rows][256], 2-byte aligned
+  ConstLdsBytes e;   // u16[n_rows][256], 2-byte aligned
 };
 
-DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte) {
-  uint16_t v;
-  __builtin_memcpy(&v, static_cast<const uint8_t*>(__builtin_assume_aligned(r.e, 2)) + (row * 256u + byte) * 2u, 2);
-  return v;
-}
+DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte);
 
 // Hierarchical lookup of the code whose first 32 bits are `top` (first bit in
 // bit 31), continued from the root row's entry `e` for the first byte.  A value
@@ -193,14 +201,37 @@ DF11_HD void store_as(void* p, const T& v) {
   __builtin_memcpy(__builtin_assume_aligned(p, alignof(T)), &v, sizeof(T));
 }
 
+// The same for workgroup memory; p is aligned to alignof(T).
+#if defined(__HIP_DEVICE_COMPILE__)
+#define DF11_LDS_ALIGNED(p, n) __builtin_assume((reinterpret_cast<uintptr_t>(p) & ((n) - 1)) == 0)
+#else
+#define DF11_LDS_ALIGNED(p, n) ((void)0)
+#endif
+template <class T>
+DF11_HD T lds_load(ConstLdsBytes p) {
+  DF11_LDS_ALIGNED(p, alignof(T));
+  T v;
+  __builtin_memcpy(&v, p, sizeof(T));
+  return v;
+}
+template <class T>
+DF11_HD void lds_store(LdsBytes p, const T& v) {
+  DF11_LDS_ALIGNED(p, alignof(T));
+  __builtin_memcpy(p, &v, sizeof(T));
+}
+
+DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte) {
+  return lds_load<uint16_t>(r.e + (row * 256u + byte) * 2u);
+}
+
 struct Tables {
-  const uint8_t* dec;     // u32[2048][2], 8-byte aligned
-  const uint8_t* cntt;    // u8[2048]
+  ConstLdsBytes dec;     // u32[2048][2], 8-byte aligned
+  ConstLdsBytes cntt;    // u8[2048]
 };
 
 // Unaligned 32-/16-bit stores (LDS supports them on gfx950; one instruction each).
-DF11_HD void store32(uint8_t* p, uint32_t v) { __builtin_memcpy(p, &v, 4); }
-DF11_HD void store16(uint8_t* p, uint32_t v) {
+DF11_HD void store32(LdsBytes p, uint32_t v) { __builtin_memcpy(p, &v, 4); }
+DF11_HD void store16(LdsBytes p, uint32_t v) {
   const uint16_t h = (uint16_t)v;
   __builtin_memcpy(p, &h, 2);
 }
@@ -240,7 +271,7 @@ DF11_HD uint32_t count_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   uint32_t cn = gap;                    // byte 0: bits consumed; bits 8 and up: codes counted
   while ((cn & 0xffu) <= 64u - (uint32_t)kK) {
-    uint32_t meta = load_as<uint32_t>(t.dec + dec_offset(w) + 4u);
+    uint32_t meta = lds_load<uint32_t>(t.dec + dec_offset(w) + 4u);
     if (meta == 0u) {
       uint32_t s, n;
       walk(l, top_bits(w, next, cn & 0xffu), s, n);
@@ -263,7 +294,7 @@ DF11_HD uint32_t count_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32
 // are gathered in a register and stored exactly, so nothing is ever written at
 // or beyond p + remaining.
 DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo, uint32_t next,
-                        uint32_t gap, uint32_t remaining, uint8_t* p) {
+                        uint32_t gap, uint32_t remaining, LdsBytes p) {
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   uint32_t c = gap;                     // bit 7 is set once the look-ahead has been appended
   uint32_t rem = remaining;
@@ -273,7 +304,7 @@ DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo
       c += 128u;
       DF11_KEEP_BRANCH();
     }
-    const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+    const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
     uint32_t syms = e.x, meta = e.y;
     if (meta == 0u) {
       uint32_t n;
@@ -295,7 +326,7 @@ DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo
         w |= (uint64_t)next << (c - 32u);
         c += 128u;
       }
-      const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+      const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
       if (meta == 0u) {
         uint32_t n;
@@ -342,7 +373,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
   for (int i = 0; i < kMainSlots; ++i) {
     r.syms[i] = 0;
     if (c <= 64u - (uint32_t)kK) {          // the lookup stays inside the chunk
-      const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+      const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
       if (meta == 0u) {
         uint32_t len;
@@ -368,7 +399,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
   for (int i = 0; i < kTailSlots; ++i) {
     r.syms[kMainSlots + i] = 0;
     if (todo) {
-      const U32x2 e = load_as<U32x2>(t.dec + dec_offset(w));
+      const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
       if (meta == 0u) {
         uint32_t len;
@@ -394,8 +425,9 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
 // atomic without return: it costs the same as an aligned store, where a store
 // to an address that is not a multiple of four stalls the LDS pipeline for
 // dozens of cycles.
-DF11_HD void or32_aligned(uint8_t* p, uint32_t v) {
-  uint32_t* w = static_cast<uint32_t*>(__builtin_assume_aligned(p, 4));
+DF11_HD void or32_aligned(LdsBytes p, uint32_t v) {
+  typedef uint32_t __attribute__((may_alias)) Word;
+  DF11_LDS Word* w = reinterpret_cast<DF11_LDS Word*>(p);
 #if defined(__HIP_DEVICE_COMPILE__)
   __hip_atomic_fetch_or(w, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 #else
@@ -408,12 +440,12 @@ DF11_HD void or32_aligned(uint8_t* p, uint32_t v) {
 // aligned words, shifted to their byte position; the unused bytes of a lookup
 // are zero and leave their neighbours alone, so no lookup needs trimming and the
 // lanes of a wavefront may write the bytes of one word in any order.
-DF11_HD void replay_chunk(const ChunkSyms& r, uint8_t* stage, uint32_t at) {
+DF11_HD void replay_chunk(const ChunkSyms& r, LdsBytes stage, uint32_t at) {
   uint32_t bit = at * 8u;
 #pragma unroll
   for (int i = 0; i < kSlots; ++i) {
     const uint64_t v = (uint64_t)r.syms[i] << (bit & 24u);
-    uint8_t* w = stage + ((bit >> 3) & ~3u);
+    LdsBytes w = stage + ((bit >> 3) & ~3u);
     or32_aligned(w, (uint32_t)v);
     or32_aligned(w + 4, (uint32_t)(v >> 32));
     bit += ((r.ks >> (3 * i)) & 7u) * 8u;
@@ -577,14 +609,14 @@ DF11_HD U32x4 merge8(const U32x2& e, const U32x2& m) {
 }
 
 // Body group g: 8 staging bytes + 8 sign|mantissa bytes `m` -> 16 bytes of BF16.
-DF11_HD void stream_group(uint32_t g, const SubPlan& p, const uint8_t* stage, const U32x2& m,
+DF11_HD void stream_group(uint32_t g, const SubPlan& p, ConstLdsBytes stage, const U32x2& m,
                           uint16_t* out) {
   const uint32_t s0 = g * (uint32_t)kGroup;
-  store_as<U32x4>(out + p.a0 + s0, merge8(load_as<U32x2>(stage + s0), m));
+  store_as<U32x4>(out + p.a0 + s0, merge8(lds_load<U32x2>(stage + s0), m));
 }
 
 // One element of a head or tail (or of everything, for unaligned buffers).
-DF11_HD void stream_element(uint32_t i, const SubPlan& p, const uint8_t* stage,
+DF11_HD void stream_element(uint32_t i, const SubPlan& p, ConstLdsBytes stage,
                             const uint8_t* sign_mantissa, uint16_t* out) {
   out[p.a0 + i] = merge(stage[i], sign_mantissa[p.a0 + i]);
 }

@@ -42,6 +42,7 @@ inline int hip_fail(hipError_t e) {
 }
 
 constexpr int kWavesPerGroup = kThreads / kLanes;   // 8
+constexpr int kLdsSkip = 16;   // decode_kernel's LDS layout starts at this address of the workgroup's allocation
 
 // ---------------------------------------------------------------------------
 // Wavefront inclusive scan with DPP (row shifts inside rows of 16 lanes, then
@@ -127,11 +128,11 @@ __global__ __launch_bounds__(kThreads) void index_kernel(const IndexArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_rows = min(a.n_luts - 1, kMaxDecodeRows);
-  uint8_t* lds_tables = lds;
+  const LdsBytes lds_tables = (LdsBytes)lds;
   uint32_t* wave_sums = reinterpret_cast<uint32_t*>(lds + kTablesBytes);
   {
     const uint4* src = reinterpret_cast<const uint4*>(a.ws + kWsTablesOffset);
-    uint4* dst = reinterpret_cast<uint4*>(lds_tables);
+    uint4* dst = reinterpret_cast<uint4*>(lds);
     for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) dst[i] = src[i];
   }
   __syncthreads();
@@ -283,13 +284,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
     const uint8_t* __restrict__ luts, const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
     uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
-  extern __shared__ __align__(16) uint8_t lds[];
+  // This kernel has no static LDS, so its dynamic LDS starts at address 0 of the
+  // workgroup's allocation (the host checks the kernel's static size before the
+  // first launch).  Spelling the base as a constant instead of the symbol of an
+  // extern array lets the compiler fold it into the offset field of every LDS
+  // instruction: the symbol costs one vector add per table lookup and staging
+  // access.  The first kLdsSkip bytes stay unused (address 0 would read as null).
+  const LdsBytes lds = reinterpret_cast<LdsBytes>((uintptr_t)kLdsSkip);
   const int tid = threadIdx.x;
   const uint32_t lane = tid & 63;
   const uint32_t wave = uniform(tid >> 6);
   const int n_rows = min(z.n_luts - 1, kMaxDecodeRows);
-  uint8_t* lds_tables = lds;
-  uint8_t* stage = lds + tables_bytes(n_rows) + wave * (uint32_t)z.stage_cap;
+  const LdsBytes lds_tables = lds;
+  const LdsBytes stage = lds + tables_bytes(n_rows) + wave * (uint32_t)z.stage_cap;
   const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
   // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
   // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
@@ -305,12 +312,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
   if (sub < z.n_subs) cur = fetch_sub(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
   {
     const uint4* src = reinterpret_cast<const uint4*>(ws + kWsTablesOffset);
-    uint4* dst = reinterpret_cast<uint4*>(lds_tables);
-    for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) dst[i] = src[i];
+    for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) lds_store<uint4>(lds_tables + 16 * i, src[i]);
   }
   // Replayed symbols are ORed into the staging area, which therefore starts out
   // zero and is cleared again after every sub-block.
-  for (uint32_t i = lane * 8u; i < (uint32_t)z.stage_cap; i += kLanes * 8u) store_as<U32x2>(stage + i, U32x2{0, 0});
+  for (uint32_t i = lane * 8u; i < (uint32_t)z.stage_cap; i += kLanes * 8u) lds_store<U32x2>(stage + i, U32x2{0, 0});
   __syncthreads();   // the only workgroup barrier: tables are read-only from here on
 
   const Tables t{lds_tables + kDecOffset, lds_tables + kCntTailOffset};
@@ -421,7 +427,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
         const uint32_t gk = g + (uint32_t)(kLanes * k);
         const bool on = (k > 0 || lane >= skew) && gk < sp.body_end;
         const uint32_t s0 = (on ? gk : 0u) * (uint32_t)kGroup;   // in range for idle lanes too
-        o[k] = merge8(load_as<U32x2>(stage + s0), m[k]);
+        o[k] = merge8(lds_load<U32x2>(stage + s0), m[k]);
       }
       const bool is_head = lane < (uint32_t)kGroup;
       const uint32_t edge = is_head ? sp.head_begin + lane : sp.tail_begin + lane - (uint32_t)kGroup;
@@ -436,13 +442,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
       // the groups past the prefetched ones
       for (g += (uint32_t)(kLanes * kPrefetchGroups); g < sp.body_end; g += kLanes) {
         const uint32_t s0 = g * (uint32_t)kGroup;
-        store_stream(out0 + s0, merge8(load_as<U32x2>(stage + s0), load_as<U32x2>(sm0 + s0)));
+        store_stream(out0 + s0, merge8(lds_load<U32x2>(stage + s0), load_as<U32x2>(sm0 + s0)));
       }
     } else if (vec_ok) {
       for (uint32_t i = sp.head_begin + lane; i < sp.head_end; i += kLanes) out0[i] = merge(stage[i], sm0[i]);
       for (uint32_t g = sp.body_begin + lane; g < sp.body_end; g += kLanes) {
         const uint32_t s0 = g * (uint32_t)kGroup;
-        store_stream(out0 + s0, merge8(load_as<U32x2>(stage + s0), load_as<U32x2>(sm0 + s0)));
+        store_stream(out0 + s0, merge8(lds_load<U32x2>(stage + s0), load_as<U32x2>(sm0 + s0)));
       }
       for (uint32_t i = sp.tail_begin + lane; i < sp.tail_end; i += kLanes) out0[i] = merge(stage[i], sm0[i]);
     } else {
@@ -454,7 +460,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))
     // sub-block's replay; the fence keeps the compiler from reordering them.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    for (uint32_t i = lane * 8u; i < stage_used(p); i += kLanes * 8u) store_as<U32x2>(stage + i, U32x2{0, 0});
+    for (uint32_t i = lane * 8u; i < stage_used(p); i += kLanes * 8u) lds_store<U32x2>(stage + i, U32x2{0, 0});
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     cur = nxt;
@@ -485,6 +491,12 @@ int device_info(DeviceInfo& info) {
     int cus = 0;
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return hip_fail(e);
+    // decode_kernel addresses its LDS from a constant base, which holds only as
+    // long as the kernel has no static LDS of its own
+    hipFuncAttributes attr;
+    e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(decode_kernel));
+    if (e != hipSuccess) return hip_fail(e);
+    if (attr.sharedSizeBytes != 0) return DF11_ERR_UNSUPPORTED;
     cache[dev].cus = cus;
     cache[dev].ok = true;
   }
@@ -556,7 +568,8 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
 
   // LDS: tables, the fused LUT rows that exist, one staging area per wavefront
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
-  const size_t lds_bytes = (size_t)tables_bytes(n_rows) + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
+  const size_t lds_bytes = (size_t)kLdsSkip + (size_t)tables_bytes(n_rows) +
+                           (size_t)kWavesPerGroup * (size_t)z.stage_cap;
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
