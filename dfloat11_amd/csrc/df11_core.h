@@ -41,8 +41,8 @@ constexpr int kTableEntries = 1 << kK;
 //                      11-bit window, first code in byte 0;
 //                      word 1 ("meta"): bits consumed in byte 0, code count in
 //                      byte 1; 0 = the first code is longer than 11 bits
-//                      when the first code is longer than 11 bits, word 0 holds the
-//                      fused entry (below) of the root row for the window's first byte
+//                      when the first code is longer than 11 bits, word 0 says where
+//                      its hierarchical lookup starts (start_of_unsettled)
 //   cntt u8[2048]      index (1<<r)|v, v = the next r bits (r < 11): how many codes
 //                      start inside those r bits
 //   rows u16[n_rows][256]  the byte LUT rows fused with the length row: bits 0-7 the
@@ -76,31 +76,6 @@ DF11_HD uint16_t make_row_entry(const Luts& l, uint32_t row, uint32_t byte) {
   if (n > 127u) n = 127u;                      // a valid length is at most 32; keeps bit 15 for the flag
   const bool names_row = d >= 240u && 256u - d < (uint32_t)l.n_rows;
   return (uint16_t)(d | ((n ? n : 1u) << 8) | (names_row ? kRowPointer : 0u));
-}
-
-// The fused rows as the decode reads them (LDS on the device).
-struct Rows {
-  ConstLdsBytes e;   // u16[n_rows][256], 2-byte aligned
-};
-
-DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte);
-
-// Hierarchical lookup of the code whose first 32 bits are `top` (first bit in
-// bit 31), continued from the root row's entry `e` for the first byte.  A value
-// >= 240 on the first three levels names row 256 - value when that row exists;
-// on the fourth level it is a symbol.
-DF11_HD void walk_from(const Rows& r, uint32_t e, uint32_t top, uint32_t& sym, uint32_t& len) {
-#pragma unroll
-  for (int level = 1; level <= 3; ++level) {
-    if (!(e & kRowPointer)) break;
-    e = row_entry(r, 256u - (e & 0xffu), (top >> (24 - 8 * level)) & 0xffu);
-  }
-  sym = e & 0xffu;
-  len = (e >> 8) & 0x7fu;
-}
-
-DF11_HD void walk(const Rows& r, uint32_t top, uint32_t& sym, uint32_t& len) {
-  walk_from(r, row_entry(r, 0u, top >> 24), top, sym, len);
 }
 
 // ---- table construction (one entry per call) --------------------------------
@@ -149,6 +124,42 @@ DF11_HD bool resolve(const Luts& l, uint64_t window, uint32_t known, uint32_t& s
   return false;
 }
 
+// Where the hierarchical lookup may start for an 11-bit window `idx` that settles
+// no code (so every code word that begins with these bits is longer than 11
+// bits): byte offset of a fused row in bits 0-15, the code byte that indexes it in
+// bits 16-17.  From the root the lookup follows a pointer per level; a level
+// can be skipped ahead of time when every slot the unknown bits can select
+// either holds one and the same pointer or is a symbol whose recorded length does
+// not belong to that level (8*level+1 .. 8*level+8): such a slot is filling that
+// no code word owns, so every code word with these leading bits goes through
+// that pointer.  Codes that pad a stem with fixed bits (the long codes given to
+// exponents >= 240) then need one row read instead of three.
+DF11_HD uint32_t start_of_unsettled(const Luts& l, uint32_t idx) {
+  uint32_t row = 0, level = 0;
+  while (level < 3u) {
+    const int known = kK - 8 * (int)level;                       // bits of this level's byte that idx fixes
+    const uint32_t kb = known >= 8 ? 8u : known > 0 ? (uint32_t)known : 0u;
+    const uint32_t lo = kb ? ((idx >> (kK - 8 * (int)level - (int)kb)) & ((1u << kb) - 1u)) << (8u - kb) : 0u;
+    const uint32_t n = 1u << (8u - kb);
+    uint32_t pointer = 0;                                        // the one pointer seen, 0 = none yet
+    bool skip = true;
+    for (uint32_t j = lo; j < lo + n; ++j) {
+      const uint32_t d = l.rows[row * 256u + j];
+      if (d >= 240u && 256u - d < (uint32_t)l.n_rows) {
+        if (pointer && pointer != d) skip = false;
+        pointer = d;
+      } else {
+        const uint32_t len = l.rows[(uint32_t)l.n_rows * 256u + d];
+        if (len > 8u * level && len <= 8u * level + 8u) skip = false;   // may be a code word's own slot
+      }
+    }
+    if (!skip || !pointer) break;
+    row = 256u - pointer;
+    ++level;
+  }
+  return (row * (uint32_t)kRowBytes) | (level << 16);
+}
+
 DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_t& meta) {
   const uint64_t window = (uint64_t)idx << (64 - kK);
   uint32_t pos = 0, k = 0;
@@ -161,7 +172,7 @@ DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_
     ++k;
   }
   meta = k ? (pos | (k << 8)) : 0u;
-  if (!k) syms = make_row_entry(l, 0u, idx >> (kK - 8));   // where the hierarchical lookup starts
+  if (!k) syms = start_of_unsettled(l, idx);
 }
 
 DF11_HD uint8_t make_cnt_tail_entry(const Luts& l, uint32_t idx) {
@@ -220,9 +231,39 @@ DF11_HD void lds_store(LdsBytes p, const T& v) {
   __builtin_memcpy(p, &v, sizeof(T));
 }
 
+// The fused rows as the decode reads them (LDS on the device).
+struct Rows {
+  ConstLdsBytes e;   // u16[n_rows][256], 2-byte aligned
+};
+
 DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte) {
   return lds_load<uint16_t>(r.e + (row * 256u + byte) * 2u);
 }
+
+// Hierarchical lookup of the code whose first 32 bits are `top` (first bit in
+// bit 31), started at byte `start >> 16` (0..3) of the code in the row at byte
+// offset `start & 0xffff` of the fused rows.  A value >= 240 on the first three
+// levels names row 256 - value when that row exists; on the fourth level it is
+// a symbol.  start = 0 is the lookup from the root as the reference does it;
+// the table entry of an 11-bit window that settles no code holds a start
+// further down where that is safe (start_of_unsettled).
+DF11_HD void walk_from(const Rows& r, uint32_t start, uint32_t top, uint32_t& sym, uint32_t& len) {
+  uint32_t level = start >> 16;
+  uint32_t shift = 24u - 8u * level;
+  uint32_t e = lds_load<uint16_t>(r.e + (start & 0xffffu) + ((top >> shift) & 0xffu) * 2u);
+  while (level < 3u && (e & kRowPointer)) {
+    ++level;
+    shift -= 8u;
+    e = row_entry(r, 256u - (e & 0xffu), (top >> shift) & 0xffu);
+  }
+  sym = e & 0xffu;
+  len = (e >> 8) & 0x7fu;
+}
+
+DF11_HD void walk(const Rows& r, uint32_t top, uint32_t& sym, uint32_t& len) {
+  walk_from(r, 0u, top, sym, len);
+}
+
 
 struct Tables {
   ConstLdsBytes dec;     // u32[2048][2], 8-byte aligned
@@ -274,7 +315,7 @@ DF11_HD uint32_t count_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32
     uint32_t meta = lds_load<uint32_t>(t.dec + dec_offset(w) + 4u);
     if (meta == 0u) {
       uint32_t s, n;
-      walk(l, top_bits(w, next, cn & 0xffu), s, n);
+      walk_from(l, lds_load<uint32_t>(t.dec + dec_offset(w)), top_bits(w, next, cn & 0xffu), s, n);
       meta = n | 0x100u;
       DF11_KEEP_BRANCH();
     }
