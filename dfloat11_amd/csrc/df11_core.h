@@ -126,8 +126,8 @@ DF11_HD bool resolve(const Luts& l, uint64_t window, uint32_t known, uint32_t& s
 
 // Where the hierarchical lookup may start for an 11-bit window `idx` that settles
 // no code (so every code word that begins with these bits is longer than 11
-// bits): byte offset of a fused row in bits 0-15, the code byte that indexes it in
-// bits 16-17.  From the root the lookup follows a pointer per level; a level
+// bits): byte offset of a fused row in bits 0-15, and in bits 16-20 the position
+// (24, 16, 8 or 0) in the code's first 32 bits of the byte that indexes that row.  From the root the lookup follows a pointer per level; a level
 // can be skipped ahead of time when every slot the unknown bits can select
 // either holds one and the same pointer or is a symbol whose recorded length does
 // not belong to that level (8*level+1 .. 8*level+8): such a slot is filling that
@@ -157,7 +157,7 @@ DF11_HD uint32_t start_of_unsettled(const Luts& l, uint32_t idx) {
     row = 256u - pointer;
     ++level;
   }
-  return (row * (uint32_t)kRowBytes) | (level << 16);
+  return (row * (uint32_t)kRowBytes) | ((24u - 8u * level) << 16);
 }
 
 DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_t& meta) {
@@ -241,27 +241,34 @@ DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte) {
 }
 
 // Hierarchical lookup of the code whose first 32 bits are `top` (first bit in
-// bit 31), started at byte `start >> 16` (0..3) of the code in the row at byte
-// offset `start & 0xffff` of the fused rows.  A value >= 240 on the first three
+// bit 31), started in the row at byte offset `start & 0xffff` of the fused rows,
+// which the code's byte at bits [start >> 16, +8) of `top` indexes (24 = first
+// byte of the code, 0 = fourth).  A value >= 240 on the first three
 // levels names row 256 - value when that row exists; on the fourth level it is
-// a symbol.  start = 0 is the lookup from the root as the reference does it;
+// a symbol.  start = 24 << 16 is the lookup from the root as the reference does it;
 // the table entry of an 11-bit window that settles no code holds a start
 // further down where that is safe (start_of_unsettled).
+DF11_HD uint32_t byte_at(uint32_t word, uint32_t shift) {   // bits [shift, shift + 8) of word
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_ubfe(word, shift, 8u);
+#else
+  return (word >> shift) & 0xffu;
+#endif
+}
+
 DF11_HD void walk_from(const Rows& r, uint32_t start, uint32_t top, uint32_t& sym, uint32_t& len) {
-  uint32_t level = start >> 16;
-  uint32_t shift = 24u - 8u * level;
-  uint32_t e = lds_load<uint16_t>(r.e + (start & 0xffffu) + ((top >> shift) & 0xffu) * 2u);
-  while (level < 3u && (e & kRowPointer)) {
-    ++level;
+  uint32_t shift = start >> 16;                  // 24 - 8 * (code byte that indexes the start row)
+  uint32_t e = lds_load<uint16_t>(r.e + (start & 0xffffu) + byte_at(top, shift) * 2u);
+  while (shift != 0u && (e & kRowPointer)) {
     shift -= 8u;
-    e = row_entry(r, 256u - (e & 0xffu), (top >> shift) & 0xffu);
+    e = row_entry(r, 256u - (e & 0xffu), byte_at(top, shift));
   }
   sym = e & 0xffu;
   len = (e >> 8) & 0x7fu;
 }
 
 DF11_HD void walk(const Rows& r, uint32_t top, uint32_t& sym, uint32_t& len) {
-  walk_from(r, 0u, top, sym, len);
+  walk_from(r, 24u << 16, top, sym, len);
 }
 
 

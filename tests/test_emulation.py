@@ -222,9 +222,10 @@ def _check_fused_rows(luts, codec=None):
     assert np.array_equal(_host_fused_rows(luts), want)
     dec, _ = _host_tables(luts)
     unresolved = np.nonzero(dec[:, 1] == 0)[0]
-    rows, levels = (dec[unresolved, 0] & 0xFFFF) // 512, dec[unresolved, 0] >> 16
-    assert (dec[unresolved, 0] & 0xFFFF).max(initial=0) % 512 == 0
-    assert (rows < n_rows).all() and (levels <= 3).all() and (dec[unresolved, 0] >> 18 == 0).all()
+    rows, shifts = (dec[unresolved, 0] & 0xFFFF) // 512, dec[unresolved, 0] >> 16
+    assert ((dec[unresolved, 0] & 0xFFFF) % 512 == 0).all()
+    assert (rows < n_rows).all() and np.isin(shifts, (24, 16, 8, 0)).all()
+    levels = (24 - shifts) // 8
     if codec is None:
         return
     start = {int(i): (int(r), int(lv)) for i, r, lv in zip(unresolved, rows, levels)}
