@@ -280,7 +280,9 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void decode_kernel(
+// Six wavefronts per SIMD is what the launch makes resident (three workgroups of
+// eight wavefronts on the four SIMDs of a CU), so registers are budgeted for six.
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void decode_kernel(
     const uint8_t* __restrict__ luts, const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
     uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
