@@ -97,8 +97,8 @@ def side_measurements(torch, dev, steps=30, warmup=30):
     matrix under each adversarial exponent distribution, and N(0, 0.02) tensors of the
     sizes a per-Linear compression produces.  Returns (mixes, sizes): name -> figures."""
     import bench_extra
-    keep = ("n_elements", "kernel_ms_median", "GBps", "hbm_frac", "bit_exact", "bits_per_exponent",
-            "max_code_bits", "compressed_over_bf16")
+    keep = ("n_elements", "kernel_ms_median", "GBps", "hbm_frac", "back_to_back_ms_per_launch",
+            "back_to_back_hbm_frac", "bit_exact", "bits_per_exponent", "max_code_bits", "compressed_over_bf16")
     mixes, sizes = {}, {}
     for kind in ("laplace", "outliers", "uniform256", "zeros"):
         w = bench_extra.make_mix(torch, kind, 4096 * 14336, dev, seed=7)

@@ -96,11 +96,24 @@ def time_decode(torch, w, steps, warmup, preheat_ms=150.0):
         ends[i].record()
     torch.cuda.synchronize()
     ms = float(np.median([s.elapsed_time(e) for s, e in zip(starts, ends)]))
+    # the same number of launches back to back, one event pair around them: what a launch
+    # costs when the next one is already queued behind it, as between the blocks of a model
+    # (an event between two launches leaves the device idle for a moment, which a kernel of
+    # a few tens of microseconds feels)
+    b0, b1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    b0.record()
+    for _ in range(steps):
+        lib.df11_decode(*args)
+    b1.record()
+    torch.cuda.synchronize()
+    ms_b2b = b0.elapsed_time(b1) / steps
     algo = algorithmic_bytes(enc.numel(), n, luts.shape[0])
     lengths = luts[-1].numpy()
     return {
         "n_elements": n, "kernel_ms_median": ms, "GBps": algo / (ms * 1e-3) / 1e9,
         "hbm_frac": algo / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "back_to_back_ms_per_launch": ms_b2b, "back_to_back_hbm_frac": algo / (ms_b2b * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "algorithmic_bytes": algo,
         "bit_exact": bool(torch.equal(out.view(torch.int16), w.flatten().view(torch.int16))),
         "bits_per_exponent": 8.0 * enc.numel() / n, "max_code_bits": int(lengths.max()),
         "distinct_exponents": int((lengths > 0).sum()), "n_luts": int(luts.shape[0]),
