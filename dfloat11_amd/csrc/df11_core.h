@@ -407,16 +407,18 @@ constexpr int kSlots = kMainSlots + kTailSlots;
 
 struct ChunkSyms {
   uint32_t syms[kSlots];   // symbol bytes of lookup i, first code in byte 0, unused bytes zero
-  uint32_t ks;             // 3 bits per lookup: how many symbols it contributes (0..4)
+  uint32_t ends[2];        // one byte per lookup 0..7: symbols of the chunk up to and including it
   uint32_t count;          // codes that start in the chunk
   bool overflow;           // ran out of slots: count and syms are incomplete
 };
+static_assert(kSlots <= 9, "ends holds the running count after lookups 0..7");
 
 DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
                                     uint32_t next, uint32_t gap) {
   ChunkSyms r;
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
-  uint32_t c = gap, n = 0, ks = 0;
+  uint32_t c = gap, n = 0;
+  r.ends[0] = r.ends[1] = 0;
 #pragma unroll
   for (int i = 0; i < kMainSlots; ++i) {
     r.syms[i] = 0;
@@ -430,12 +432,11 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
         DF11_KEEP_BRANCH();
       }
       r.syms[i] = syms;
-      const uint32_t k = meta >> 8;
-      ks |= k << (3 * i);
-      n += k;
+      n += (meta >> 8) & 0xffu;
       w <<= (meta & 63u);
       c += meta & 0xffu;
     }
+    r.ends[i >> 2] |= n << (8 * (i & 3));   // also for a lane that skipped the lookup: later ones start here
   }
   r.overflow = c <= 64u - (uint32_t)kK;
   uint32_t todo = 0;                          // codes that still start before the chunk ends
@@ -457,14 +458,13 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
       r.syms[kMainSlots + i] = syms;
       const uint32_t k = meta >> 8;
       const uint32_t take = k < todo ? k : todo;
-      ks |= take << (3 * (kMainSlots + i));
       n += take;
       todo -= take;
       w <<= (meta & 63u);
     }
+    if (kMainSlots + i < 8) r.ends[(kMainSlots + i) >> 2] |= n << (8 * ((kMainSlots + i) & 3));
   }
   r.overflow = r.overflow || todo != 0u;
-  r.ks = ks;
   r.count = n;
   return r;
 }
@@ -489,14 +489,14 @@ DF11_HD void or32_aligned(LdsBytes p, uint32_t v) {
 // are zero and leave their neighbours alone, so no lookup needs trimming and the
 // lanes of a wavefront may write the bytes of one word in any order.
 DF11_HD void replay_chunk(const ChunkSyms& r, LdsBytes stage, uint32_t at) {
-  uint32_t bit = at * 8u;
 #pragma unroll
   for (int i = 0; i < kSlots; ++i) {
-    const uint64_t v = (uint64_t)r.syms[i] << (bit & 24u);
-    LdsBytes w = stage + ((bit >> 3) & ~3u);
+    // lookup i starts where the lookups before it end
+    const uint32_t pos = i == 0 ? at : at + ((r.ends[(i - 1) >> 2] >> (8 * ((i - 1) & 3))) & 0xffu);
+    const uint64_t v = (uint64_t)r.syms[i] << ((pos & 3u) * 8u);
+    LdsBytes w = stage + (pos & ~3u);
     or32_aligned(w, (uint32_t)v);
     or32_aligned(w + 4, (uint32_t)(v >> 32));
-    bit += ((r.ks >> (3 * i)) & 7u) * 8u;
   }
 }
 

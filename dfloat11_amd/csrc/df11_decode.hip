@@ -298,7 +298,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))
   const uint32_t wave = uniform(tid >> 6);
   const int n_rows = min(z.n_luts - 1, kMaxDecodeRows);
   const LdsBytes lds_tables = lds;
-  const LdsBytes stage = lds + tables_bytes(n_rows) + wave * (uint32_t)z.stage_cap;
+  const uint32_t stage_offset = (uint32_t)tables_bytes(n_rows) + wave * (uint32_t)z.stage_cap;   // multiple of 16
+  const LdsBytes stage = lds + stage_offset;
   const uint32_t* __restrict__ subpos = reinterpret_cast<const uint32_t*>(ws + kWsSubposOffset);
   // Lane constants of the 5-bit gap: two bytes starting at gap_byte hold it,
   // gap_shift positions it.  Lane 63's field ends its sub-block's gap bytes, so
@@ -397,7 +398,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))
     const SubPlan p = plan_sub((int64_t)base, total, z.n_elements, z.stage_cap);   // uniform
     const uint32_t quota = thread_quota(excl, count, p.n_out);
     if (all_fit && wave_all(quota == count))
-      replay_chunk(cs, stage, p.phase + excl);
+      replay_chunk(cs, lds, stage_offset + p.phase + excl);   // one base for all: the wavefront's offset rides in the index
     else
       emit_chunk(t, l, c.hi, c.lo, c.next, gap, quota, stage + p.phase + excl);
     // Staging is exchanged between the lanes of one wavefront only; its LDS
