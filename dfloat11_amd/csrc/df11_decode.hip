@@ -71,7 +71,8 @@ __device__ __forceinline__ uint32_t wave_total(uint32_t inclusive) {
   return (uint32_t)__builtin_amdgcn_readlane((int)inclusive, 63);
 }
 
-// Copies the byte LUT rows a pointer can reach, then the length row, into LDS.
+// Copies the byte LUT rows a pointer can reach, then the length row, into LDS
+// (table construction reads them; the decode reads the fused rows it writes).
 __device__ __forceinline__ void stage_rows(const uint8_t* __restrict__ luts, int n_luts, int n_rows,
                                            uint8_t* rows, int tid, int n_threads) {
   for (int i = tid; i < n_rows * 256; i += n_threads) rows[i] = luts[i];
@@ -112,7 +113,6 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const uint8_t* __rest
 // the block's own output position.
 // ---------------------------------------------------------------------------
 struct IndexArgs {
-  const uint8_t* luts;
   const uint8_t* codes;
   const uint32_t* positions;
   const uint8_t* gaps;
@@ -283,7 +283,7 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
 // Six wavefronts per SIMD is what the launch makes resident (three workgroups of
 // eight wavefronts on the four SIMDs of a CU), so registers are budgeted for six.
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void decode_kernel(
-    const uint8_t* __restrict__ luts, const uint8_t* __restrict__ codes,
+    const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
     uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
   // This kernel has no static LDS, so its dynamic LDS starts at address 0 of the
@@ -530,7 +530,6 @@ int enqueue_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const 
   if (e != hipSuccess) return hip_fail(e);
   if (n_blocks > 0) {
     IndexArgs a;
-    a.luts = luts;
     a.codes = encoded_exponent;
     a.positions = output_positions;
     a.gaps = gaps;
@@ -577,7 +576,8 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
 
-  hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, luts,
+  (void)luts;   // read by df11_prepare only: the decode finds them fused in the workspace
+  hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s,
                      encoded_exponent, sign_mantissa, gaps, outputs, ws, z);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? DF11_OK : hip_fail(e);
