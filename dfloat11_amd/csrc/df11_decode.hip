@@ -617,7 +617,7 @@ int scratch_of_current_device(uint8_t** out) {
 
 extern "C" {
 
-int df11_version(void) { return 2; }
+int df11_version(void) { return 3; }
 
 const char* df11_error_string(int code) {
   switch (code) {

@@ -39,6 +39,7 @@ extern "C" {
 #define DF11_SUBBLOCK_BYTES 512
 #define DF11_MAX_ELEMS_PER_SUBBLOCK 4096
 
+/* Version of this interface: 3 = df11_decode_static_workspace added, workspace holds fused LUT rows. */
 int df11_version(void);
 const char *df11_error_string(int code);
 

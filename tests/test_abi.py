@@ -24,7 +24,7 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_error_strings():
     hip = _native.hip_lib()
-    assert hip.df11_version() == 2
+    assert hip.df11_version() == 3
     assert hip.df11_error_string(0) == b"ok"
     assert hip.df11_error_string(-1) == b"invalid argument"
     # header + tables + 17 fused LUT rows + (8 sub-blocks per 4096-byte block + 1) positions, rounded to 16
