@@ -295,7 +295,7 @@ def main():
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": profiled_traffic(),
-                     "kernel": "decode_kernel", "avg_launch_ms": avg_kernel_ms},
+                     "kernel": "decode_kernel_deep", "avg_launch_ms": avg_kernel_ms},
     }
     if not a.no_mixes:
         copies.clear()

@@ -224,12 +224,11 @@ struct DecodeSizes {
   int32_t vec_ok;         // sign_mantissa 8-byte aligned and out 16-byte aligned
 };
 
-// Body groups per lane whose sign|mantissa bytes are requested a whole decode
-// early; the remaining groups of a sub-block (about a third for typical weights)
-// load theirs between the stores.  Measured on MI355X: 2 -> 140 us, 3 -> 145 us,
-// 4 -> 153 us, 1 -> 145 us for the 218 M element block; the memory system does
-// better with loads and stores interleaved than with long bursts of either.
-constexpr int kPrefetchGroups = 2;
+// kPrefetch (template parameter of the decode body): body groups per lane whose
+// sign|mantissa bytes are requested a whole decode early; the remaining groups of
+// a sub-block load theirs between the stores.  How many to request early and how
+// many wavefronts to keep resident go together and depend on the stream (see the
+// launch plans next to the kernels).
 constexpr int kBatchAlignGroups = 16;   // batches of 64 groups start on multiples of 16 groups (256 B of output)
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) {
@@ -280,13 +279,12 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-// Six wavefronts per SIMD is what the launch makes resident (three workgroups of
-// eight wavefronts on the four SIMDs of a CU), so registers are budgeted for six.
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void decode_kernel(
+template <int kPrefetchGroups>
+__device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
     uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
-  // This kernel has no static LDS, so its dynamic LDS starts at address 0 of the
+  // The decode kernels have no static LDS, so its dynamic LDS starts at address 0 of the
   // workgroup's allocation (the host checks the kernel's static size before the
   // first launch).  Spelling the base as a constant instead of the symbol of an
   // extern array lets the compiler fold it into the offset field of every LDS
@@ -470,6 +468,57 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))
   }
 }
 
+// Launch plans.  The kernel is one body compiled three ways; which one runs is
+// decided per stream at launch time from two numbers the host knows, the number of
+// sub-blocks and the elements an average sub-block produces.  Measured on MI355X
+// (N(0, 0.02), Laplace, one-bit and incompressible streams of 17 M to 622 M
+// elements):
+//   wide     3 workgroups per CU (6 wavefronts per SIMD), 2 groups requested early.
+//            Best when wavefronts are the scarce resource: streams of fewer than
+//            about 38 M elements (a few rounds of sub-blocks: the launch is
+//            latency-bound) and streams whose decode is bound by vector
+//            instructions (long codes, few elements per sub-block).
+//   deep     2 workgroups per CU (4 per SIMD), 3 groups requested early: a typical
+//            sub-block is 3 groups per lane, so the whole write-out runs on bytes
+//            that are already there.  Fewer, deeper memory streams: 1 % (218 M
+//            elements) to 6-8 % (622 M) faster than `wide` on weight-like streams.
+//   deepest  2 workgroups per CU, 6 groups requested early, for streams of short
+//            codes (a sub-block of one-bit codes is 8 groups per lane): 74 % of the
+//            HBM peak on the all-zero mix against 68 % with `wide`.
+// The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
+#define DF11_DECODE_KERNEL(name, prefetch, waves_per_simd)                                        \
+  __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
+                                                                             waves_per_simd)))    \
+  void name(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,         \
+            const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,                         \
+            const uint8_t* __restrict__ ws, const DecodeSizes z) {                                \
+    decode_body<prefetch>(codes, sign_mantissa, gaps, out, ws, z);                                \
+  }
+DF11_DECODE_KERNEL(decode_kernel_wide, 2, 6)
+DF11_DECODE_KERNEL(decode_kernel_deep, 3, 4)
+DF11_DECODE_KERNEL(decode_kernel_deepest, 6, 4)
+#undef DF11_DECODE_KERNEL
+
+typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);
+struct LaunchPlan {
+  DecodeKernel kernel;
+  int groups_per_cu;
+};
+constexpr int kWideGroupsPerCu = 3;
+constexpr int kDeepGroupsPerCu = 2;
+constexpr int kMinElemsPerWaveForDeep = 6144;  // output per resident wavefront of the wide plan: four typical sub-blocks
+constexpr int kMinElemsPerSubForDeep = 1024;   // below: more than 4 bits per exponent, decode-bound
+constexpr int kMinElemsPerSubForDeepest = 2560;
+
+LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
+  const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
+  const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
+  if (n_elements < kMinElemsPerWaveForDeep * wide_waves || elems_per_sub < kMinElemsPerSubForDeep)
+    return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu};
+  if (elems_per_sub < kMinElemsPerSubForDeepest) return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu};
+  return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu};
+}
+
 // Plain streaming copy, 16 bytes per lane: the known-traffic kernel against
 // which hardware byte counters are calibrated.
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src,
@@ -494,12 +543,14 @@ int device_info(DeviceInfo& info) {
     int cus = 0;
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return hip_fail(e);
-    // decode_kernel addresses its LDS from a constant base, which holds only as
-    // long as the kernel has no static LDS of its own
-    hipFuncAttributes attr;
-    e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(decode_kernel));
-    if (e != hipSuccess) return hip_fail(e);
-    if (attr.sharedSizeBytes != 0) return DF11_ERR_UNSUPPORTED;
+    // the decode kernels address their LDS from a constant base, which holds only
+    // as long as they have no static LDS of their own
+    for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deepest}) {
+      hipFuncAttributes attr;
+      e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(k));
+      if (e != hipSuccess) return hip_fail(e);
+      if (attr.sharedSizeBytes != 0) return DF11_ERR_UNSUPPORTED;
+    }
     cache[dev].cus = cus;
     cache[dev].ok = true;
   }
@@ -509,13 +560,10 @@ int device_info(DeviceInfo& info) {
 
 constexpr int kLdsPerCu = 160 * 1024;
 
-// Workgroups resident per CU.  Three (six wavefronts per SIMD) hide the decode
-// latency completely; a fourth only adds memory streams that compete for HBM
-// pages and measured 3 % slower; two are 8 % slower.
-constexpr int kMaxGroupsPerCu = 3;
-int groups_per_cu(size_t lds_bytes) {
+// Workgroups of lds_bytes each that fit a CU, at most `wanted`.
+int groups_per_cu(size_t lds_bytes, int wanted) {
   int n = (int)(kLdsPerCu / lds_bytes);
-  if (n > kMaxGroupsPerCu) n = kMaxGroupsPerCu;
+  if (n > wanted) n = wanted;
   return n < 1 ? 1 : n;
 }
 
@@ -540,7 +588,7 @@ int enqueue_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const 
     a.n_luts = n_luts;
     a.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
     const size_t lds_bytes = (size_t)kTablesBytes + 64;
-    int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
+    int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, kWideGroupsPerCu);
     if (grid > n_blocks) grid = n_blocks;
     hipLaunchKernelGGL(index_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s, a);
     e = hipGetLastError();
@@ -572,12 +620,13 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
   const size_t lds_bytes = (size_t)kLdsSkip + (size_t)tables_bytes(n_rows) +
                            (size_t)kWavesPerGroup * (size_t)z.stage_cap;
-  int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes);
+  const LaunchPlan plan = plan_launch(z.n_subs, n_elements, info.cus);
+  int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, plan.groups_per_cu);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
 
   (void)luts;   // read by df11_prepare only: the decode finds them fused in the workspace
-  hipLaunchKernelGGL(decode_kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s,
+  hipLaunchKernelGGL(plan.kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s,
                      encoded_exponent, sign_mantissa, gaps, outputs, ws, z);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? DF11_OK : hip_fail(e);
