@@ -25,6 +25,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "../../include/df11.h"
@@ -510,7 +511,15 @@ constexpr int kMinElemsPerWaveForDeep = 6144;  // output per resident wavefront 
 constexpr int kMinElemsPerSubForDeep = 1024;   // below: more than 4 bits per exponent, decode-bound
 constexpr int kMinElemsPerSubForDeepest = 2560;
 
+std::atomic<int> g_forced_plan{-1};   // df11_force_launch_plan: -1 = choose per stream
+
 LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
+  switch (g_forced_plan.load(std::memory_order_relaxed)) {
+    case DF11_PLAN_WIDE: return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu};
+    case DF11_PLAN_DEEP: return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu};
+    case DF11_PLAN_DEEPEST: return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu};
+    default: break;
+  }
   const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
   if (n_elements < kMinElemsPerWaveForDeep * wide_waves || elems_per_sub < kMinElemsPerSubForDeep)
@@ -714,6 +723,12 @@ int df11_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const uin
     if (e != hipSuccess) return hip_fail(e);
     *max_elems_per_subblock = (int32_t)h.max_sub_elems;
   }
+  return DF11_OK;
+}
+
+int df11_force_launch_plan(int plan) {
+  if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_DEEPEST) return DF11_ERR_INVALID_ARGUMENT;
+  g_forced_plan.store(plan, std::memory_order_relaxed);
   return DF11_OK;
 }
 

@@ -121,6 +121,20 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
                                  int32_t max_elems_per_subblock, void *stream);
 
 /*
+ * The decode kernel exists in three launch plans (workgroups resident per CU and
+ * depth of its requests for sign_mantissa bytes); df11_decode picks one per
+ * stream from its size and its elements per 512 bytes of bitstream.  This call
+ * pins the plan for every later decode of the process, or hands the choice back
+ * (DF11_PLAN_AUTO).  Testing and measurement aid with no counterpart in the
+ * reference: every plan decodes every stream to the same bits.
+ */
+#define DF11_PLAN_AUTO (-1)
+#define DF11_PLAN_WIDE 0
+#define DF11_PLAN_DEEP 1
+#define DF11_PLAN_DEEPEST 2
+int df11_force_launch_plan(int plan);
+
+/*
  * Streaming device copy of n_bytes (multiple of 16, both pointers 16-byte
  * aligned).  Measurement aid with no counterpart in the reference: a kernel of
  * known HBM traffic against which profiler byte counters are calibrated.

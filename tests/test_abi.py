@@ -70,3 +70,10 @@ def test_plain_c_caller_builds_against_the_header():
     subprocess.run(["make", "-s", "-C", d], check=True)
     out = subprocess.run(["ldd", os.path.join(d, "abi_roundtrip")], capture_output=True, text=True, check=True).stdout
     assert "libdf11_hip.so" in out and "libdf11_codec.so" in out and "not found" not in out
+
+
+def test_launch_plan_override_is_validated():
+    hip = _native.hip_lib()
+    assert hip.df11_force_launch_plan(3) == -1 and hip.df11_force_launch_plan(-2) == -1
+    for plan in (0, 1, 2, -1):
+        assert hip.df11_force_launch_plan(plan) == 0

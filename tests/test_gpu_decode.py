@@ -57,6 +57,49 @@ def test_gpu_matches_oracle(oracle, kind, n):
     assert np.array_equal(got, w)
 
 
+@pytest.fixture()
+def launch_plan():
+    """Pins one of the decode kernel's launch plans for a test and hands the choice back after it."""
+    from dfloat11_amd import _native
+    lib = _native.hip_lib()
+
+    def force(plan):
+        assert lib.df11_force_launch_plan(plan) == 0
+    yield force
+    assert lib.df11_force_launch_plan(-1) == 0
+
+
+@pytest.mark.parametrize("plan", [0, 1, 2], ids=["wide", "deep", "deepest"])
+def test_gpu_every_launch_plan_matches_oracle(oracle, launch_plan, plan):
+    """The plans differ in resident workgroups and in how many groups of sign|mantissa
+    bytes are requested early; the automatic choice sends small streams to one of them
+    only.  Pinned, each plan decodes every kind, ragged sizes, unaligned buffers and the
+    worst-case staging to the oracle's bits."""
+    launch_plan(plan)
+    for kind in KINDS:
+        for n in (1, 511, 4097, 70_001, 300_000):
+            print(f"case plan={plan} kind={kind} n={n}", flush=True)
+            w = make_case(kind, n, 211 + plan)
+            c = compress_product(w)
+            ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                                  c["output_positions"], c["gaps"])
+            assert np.array_equal(gpu_decode(c), ref), (kind, n)
+            assert np.array_equal(ref, w)
+    w = make_case("laplace", 120_000, 79)
+    c = compress_product(w)
+    for pad in (1, 4, 7):
+        assert np.array_equal(gpu_decode(c, pad_front=pad), w), pad
+    buf = torch.zeros(w.size + 16, dtype=torch.bfloat16, device=DEV)
+    for shift in (1, 3, 8):
+        buf.zero_()
+        assert np.array_equal(gpu_decode(c, out=buf[shift:shift + w.size]), w)
+        whole = buf.view(torch.int16).cpu().numpy()
+        assert not whole[:shift].any() and not whole[shift + w.size:].any()
+    for kind in ("normal", "zeros", "fib"):
+        w = make_case(kind, 200_000, 67)
+        assert np.array_equal(gpu_decode(compress_product(w), max_elems=0), w), kind
+
+
 def test_gpu_random_codes_and_fillings(oracle):
     """Random prefix codes (deep, incomplete, symbols >= 240) with the unowned LUT
     slots filled three ways, and tiny tensors over large alphabets: GPU == original
