@@ -200,17 +200,25 @@ __device__ __forceinline__ void claim(uint32_t& v, T&... rest) {
   claim(rest...);
 }
 
-// Streaming access: the bitstream and the sign|mantissa bytes are read once and
-// the output is written once, so both bypass cache retention (nontemporal).  With
-// the kernel bound by HBM this is worth about 5 % on MI355X.
+// Streaming access: the output is written once and, within one decode, the
+// bitstream and the sign|mantissa bytes are read once, so they bypass cache
+// retention (nontemporal): worth 5-8 % on a large stream (plain stores: 145 vs
+// 133 us on the 218 M-element block; plain loads: 387 vs 368 us on 622 M
+// elements).  kStreaming = false reads with plain loads instead, for the small
+// streams of the `wide` plan: what a small stream's module reads may still sit in
+// the 256 MB memory-side cache from the previous forward pass (a 17 M-element
+// weight decodes in 13.1-13.8 us instead of 14.8-15.4 us then), and when it does
+// not the plain loads cost 1.5 % (16.3 vs 16.1 us with 24 copies decoded in turn).
 typedef uint32_t V4u __attribute__((ext_vector_type(4)));
 typedef uint32_t V2u __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void store_stream(uint16_t* p, const U32x4& v) {
   const V4u x = {v.x, v.y, v.z, v.w};
   __builtin_nontemporal_store(x, reinterpret_cast<V4u*>(p));
 }
+template <bool kStreaming>
 __device__ __forceinline__ U32x2 load_stream(const uint8_t* p) {   // p 8-byte aligned
-  const V2u v = __builtin_nontemporal_load(reinterpret_cast<const V2u*>(p));
+  const V2u v = kStreaming ? __builtin_nontemporal_load(reinterpret_cast<const V2u*>(p))
+                           : *reinterpret_cast<const V2u*>(p);
   return U32x2{v.x, v.y};
 }
 
@@ -248,6 +256,7 @@ struct SubInputs {
 // Bytes [8*lane, 8*lane + 12) of sub-block `sub` (uniform), its two gap bytes and
 // its output position.  gap_byte: lane's byte offset inside the sub-block's 40
 // bytes of gaps, chosen so that byte + 1 stays inside them.
+template <bool kStreaming>
 __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes,
                                                const uint8_t* __restrict__ gaps,
                                                const uint32_t* __restrict__ subpos,
@@ -257,7 +266,7 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   const int64_t sub_off = sub * kSubBytes;                       // uniform
   if (z.codes_aligned && sub_off + kSubBytes + 4 <= z.n_bytes) {   // uniform: whole sub-block + look-ahead in range
     const uint8_t* p = codes + sub_off + lane * (uint32_t)kChunkBytes;
-    const U32x2 v = load_stream(p);
+    const U32x2 v = load_stream<kStreaming>(p);
     in.d0 = v.x;
     in.d1 = v.y;
     in.d2 = load_as<uint32_t>(p + 8);
@@ -280,7 +289,7 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-template <int kPrefetchGroups>
+template <int kPrefetchGroups, bool kStreaming>
 __device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
@@ -311,7 +320,7 @@ __device__ __forceinline__ void decode_body(
   // The first sub-block's inputs are requested before the tables are copied, so
   // that their latency overlaps with that of the copy.
   SubInputs cur{};
-  if (sub < z.n_subs) cur = fetch_sub(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
+  if (sub < z.n_subs) cur = fetch_sub<kStreaming>(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
   {
     const uint4* src = reinterpret_cast<const uint4*>(ws + kWsTablesOffset);
     for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) lds_store<uint4>(lds_tables + 16 * i, src[i]);
@@ -346,7 +355,7 @@ __device__ __forceinline__ void decode_body(
     // sub-block's inputs and this one's sign|mantissa bytes
     const int64_t next_sub = sub + stride;
     SubInputs nxt = cur;
-    if (next_sub < z.n_subs) nxt = fetch_sub(codes, gaps, subpos, z, next_sub, lane, gap_byte, vzero);
+    if (next_sub < z.n_subs) nxt = fetch_sub<kStreaming>(codes, gaps, subpos, z, next_sub, lane, gap_byte, vzero);
 
     const uint32_t base = uniform(cur.base);
     const uint32_t a0 = base & ~(uint32_t)(kGroup - 1);
@@ -366,7 +375,7 @@ __device__ __forceinline__ void decode_body(
     for (int k = 0; k < kPrefetchGroups; ++k) {
       m[k] = U32x2{0, 0};
       const uint32_t s0 = (first_body + lane + (uint32_t)(kLanes * k) - skew) * (uint32_t)kGroup;
-      if (vec_ok && (k > 0 || lane >= skew) && s0 + (uint32_t)kGroup <= hint_len) m[k] = load_stream(sm0 + s0);
+      if (vec_ok && (k > 0 || lane >= skew) && s0 + (uint32_t)kGroup <= hint_len) m[k] = load_stream<kStreaming>(sm0 + s0);
     }
     // The ragged ends, fewer than 8 elements each: lanes 0..7 take the head, lanes
     // 8..15 the tail, one element per lane, its sign|mantissa byte requested now.
@@ -474,7 +483,8 @@ __device__ __forceinline__ void decode_body(
 // sub-blocks and the elements an average sub-block produces.  Measured on MI355X
 // (N(0, 0.02), Laplace, one-bit and incompressible streams of 17 M to 622 M
 // elements):
-//   wide     3 workgroups per CU (6 wavefronts per SIMD), 2 groups requested early.
+//   wide     3 workgroups per CU (6 wavefronts per SIMD), 2 groups requested early,
+//            plain (cacheable) loads.
 //            Best when wavefronts are the scarce resource: streams of fewer than
 //            about 38 M elements (a few rounds of sub-blocks: the launch is
 //            latency-bound) and streams whose decode is bound by vector
@@ -487,17 +497,17 @@ __device__ __forceinline__ void decode_body(
 //            codes (a sub-block of one-bit codes is 8 groups per lane): 74 % of the
 //            HBM peak on the all-zero mix against 68 % with `wide`.
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
-#define DF11_DECODE_KERNEL(name, prefetch, waves_per_simd)                                        \
+#define DF11_DECODE_KERNEL(name, prefetch, streaming, waves_per_simd)                             \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
                                                                              waves_per_simd)))    \
   void name(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,         \
             const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,                         \
             const uint8_t* __restrict__ ws, const DecodeSizes z) {                                \
-    decode_body<prefetch>(codes, sign_mantissa, gaps, out, ws, z);                                \
+    decode_body<prefetch, streaming>(codes, sign_mantissa, gaps, out, ws, z);                     \
   }
-DF11_DECODE_KERNEL(decode_kernel_wide, 2, 6)
-DF11_DECODE_KERNEL(decode_kernel_deep, 3, 4)
-DF11_DECODE_KERNEL(decode_kernel_deepest, 6, 4)
+DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, 6)
+DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, 4)
 #undef DF11_DECODE_KERNEL
 
 typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);
