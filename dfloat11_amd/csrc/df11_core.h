@@ -40,9 +40,11 @@ constexpr int kTableEntries = 1 << kK;
 //   dec  u32[2048][2]  word 0: the symbols of up to four codes that end inside the
 //                      11-bit window, first code in byte 0;
 //                      word 1 ("meta"): bits consumed in byte 0, code count in
-//                      byte 1; 0 = the first code is longer than 11 bits
-//                      when the first code is longer than 11 bits, word 0 says where
-//                      its hierarchical lookup starts (start_of_unsettled)
+//                      byte 1.  When the first code is longer than 11 bits, bit 31
+//                      of word 1 is set and the two words say where the code's
+//                      hierarchical lookup starts (start_of_unsettled): word 0 the
+//                      byte offset of a fused row, bits 0-4 of word 1 the position
+//                      of the code byte that indexes it
 //   cntt u8[2048]      index (1<<r)|v, v = the next r bits (r < 11): how many codes
 //                      start inside those r bits
 //   rows u16[n_rows][256]  the byte LUT rows fused with the length row: bits 0-7 the
@@ -126,15 +128,17 @@ DF11_HD bool resolve(const Luts& l, uint64_t window, uint32_t known, uint32_t& s
 
 // Where the hierarchical lookup may start for an 11-bit window `idx` that settles
 // no code (so every code word that begins with these bits is longer than 11
-// bits): byte offset of a fused row in bits 0-15, and in bits 16-20 the position
-// (24, 16, 8 or 0) in the code's first 32 bits of the byte that indexes that row.  From the root the lookup follows a pointer per level; a level
+// bits): the byte offset of a fused row, and the position (24, 16, 8 or 0) in the
+// code's first 32 bits of the byte that indexes that row, marked with kUnsettled.
+// From the root the lookup follows a pointer per level; a level
 // can be skipped ahead of time when every slot the unknown bits can select
 // either holds one and the same pointer or is a symbol whose recorded length does
 // not belong to that level (8*level+1 .. 8*level+8): such a slot is filling that
 // no code word owns, so every code word with these leading bits goes through
 // that pointer.  Codes that pad a stem with fixed bits (the long codes given to
 // exponents >= 240) then need one row read instead of three.
-DF11_HD uint32_t start_of_unsettled(const Luts& l, uint32_t idx) {
+constexpr uint32_t kUnsettled = 0x80000000u;
+DF11_HD void start_of_unsettled(const Luts& l, uint32_t idx, uint32_t& row_offset, uint32_t& at) {
   uint32_t row = 0, level = 0;
   while (level < 3u) {
     const int known = kK - 8 * (int)level;                       // bits of this level's byte that idx fixes
@@ -157,7 +161,8 @@ DF11_HD uint32_t start_of_unsettled(const Luts& l, uint32_t idx) {
     row = 256u - pointer;
     ++level;
   }
-  return (row * (uint32_t)kRowBytes) | ((24u - 8u * level) << 16);
+  row_offset = row * (uint32_t)kRowBytes;
+  at = kUnsettled | (24u - 8u * level);
 }
 
 DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_t& meta) {
@@ -171,8 +176,8 @@ DF11_HD void make_dec_entry(const Luts& l, uint32_t idx, uint32_t& syms, uint32_
     pos += n;
     ++k;
   }
-  meta = k ? (pos | (k << 8)) : 0u;
-  if (!k) syms = start_of_unsettled(l, idx);
+  meta = pos | (k << 8);
+  if (!k) start_of_unsettled(l, idx, syms, meta);
 }
 
 DF11_HD uint8_t make_cnt_tail_entry(const Luts& l, uint32_t idx) {
@@ -236,40 +241,48 @@ struct Rows {
   ConstLdsBytes e;   // u16[n_rows][256], 2-byte aligned
 };
 
-DF11_HD uint32_t row_entry(const Rows& r, uint32_t row, uint32_t byte) {
-  return lds_load<uint16_t>(r.e + (row * 256u + byte) * 2u);
+// One fused entry, zero-extended.  The compiler is not told that the upper half is
+// zero: it would otherwise test the pointer flag on the 16-bit value and extend
+// that again for every later use.
+DF11_HD uint32_t row_entry_at(const Rows& r, uint32_t byte_offset) {
+  uint32_t e = lds_load<uint16_t>(r.e + byte_offset);
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("" : "+v"(e));
+  __builtin_assume(e < 65536u);
+#endif
+  return e;
 }
 
 // Hierarchical lookup of the code whose first 32 bits are `top` (first bit in
-// bit 31), started in the row at byte offset `start & 0xffff` of the fused rows,
-// which the code's byte at bits [start >> 16, +8) of `top` indexes (24 = first
+// bit 31), started in the row at byte offset `row_offset` of the fused rows,
+// which the code's byte at bits [at & 31, +8) of `top` indexes (24 = first
 // byte of the code, 0 = fourth).  A value >= 240 on the first three
 // levels names row 256 - value when that row exists; on the fourth level it is
-// a symbol.  start = 24 << 16 is the lookup from the root as the reference does it;
-// the table entry of an 11-bit window that settles no code holds a start
-// further down where that is safe (start_of_unsettled).
-DF11_HD uint32_t byte_at(uint32_t word, uint32_t shift) {   // bits [shift, shift + 8) of word
+// a symbol.  Row offset 0 with at = 24 is the lookup from the root as the
+// reference does it; the table entry of an 11-bit window that settles no code
+// holds a start further down where that is safe (start_of_unsettled).
+// `at` is kUnsettled | position, as the table holds it.  Returns the fused entry
+// of the symbol.
+DF11_HD uint32_t byte_at(uint32_t word, uint32_t shift) {   // bits [shift & 31, +8) of word
 #if defined(__HIP_DEVICE_COMPILE__)
-  return __builtin_amdgcn_ubfe(word, shift, 8u);
+  return __builtin_amdgcn_ubfe(word, shift, 8u);           // the instruction reads five bits of the shift
 #else
-  return (word >> shift) & 0xffu;
+  return (word >> (shift & 31u)) & 0xffu;
 #endif
 }
 
-DF11_HD void walk_from(const Rows& r, uint32_t start, uint32_t top, uint32_t& sym, uint32_t& len) {
-  uint32_t shift = start >> 16;                  // 24 - 8 * (code byte that indexes the start row)
-  uint32_t e = lds_load<uint16_t>(r.e + (start & 0xffffu) + byte_at(top, shift) * 2u);
-  while (shift != 0u && (e & kRowPointer)) {
-    shift -= 8u;
-    e = row_entry(r, 256u - (e & 0xffu), byte_at(top, shift));
+DF11_HD uint32_t walk_from(const Rows& r, uint32_t row_offset, uint32_t at, uint32_t top) {
+  uint32_t e = row_entry_at(r, row_offset + byte_at(top, at) * 2u);
+  while (at != kUnsettled && e >= kRowPointer) {
+    at -= 8u;
+    e = row_entry_at(r, ((256u - (e & 0xffu)) * 256u + byte_at(top, at)) * 2u);
   }
-  sym = e & 0xffu;
-  len = (e >> 8) & 0x7fu;
+  return e;
 }
-
-DF11_HD void walk(const Rows& r, uint32_t top, uint32_t& sym, uint32_t& len) {
-  walk_from(r, 24u << 16, top, sym, len);
-}
+DF11_HD uint32_t entry_symbol(uint32_t e) { return e & 0xffu; }
+DF11_HD uint32_t entry_length(uint32_t e) { return (e >> 8) & 0x7fu; }
+// One code of entry_length bits, as the second word of a table entry.
+DF11_HD uint32_t entry_meta(uint32_t e) { return entry_length(e) | 0x100u; }
 
 
 struct Tables {
@@ -299,11 +312,12 @@ DF11_HD uint64_t with_next(uint64_t w, uint32_t next, uint32_t c) {
 }
 
 // The next 32 stream bits at the top of window `w`, of which the 64 - c topmost
-// bits are valid chunk bits and the rest zero (c < 64); `next` holds the 32 bits
-// that follow the chunk.
-DF11_HD uint32_t top_bits(uint64_t w, uint32_t next, uint32_t c) {
-  const uint32_t hi = (uint32_t)(w >> 32);
-  return c > 32u ? hi | (next >> (64u - c)) : hi;
+// bits are valid chunk bits and the rest zero (c < 64); `next31` holds the 32 bits
+// that follow the chunk, shifted left by 31 (look_ahead): moved down by 63 - c
+// they line up with the window's first invalid bit.
+DF11_HD uint64_t look_ahead(uint32_t next) { return (uint64_t)next << 31; }
+DF11_HD uint32_t top_bits(uint64_t w, uint64_t next31, uint32_t c) {
+  return (uint32_t)((w | (next31 >> (63u - c))) >> 32);
 }
 
 // Byte offset of the table entry for the top kK bits of the window.
@@ -317,13 +331,12 @@ DF11_HD uint32_t dec_offset(uint64_t w) { return ((uint32_t)(w >> 32) >> (32 - k
 DF11_HD uint32_t count_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
                              uint32_t next, uint32_t gap) {
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
+  const uint64_t next31 = look_ahead(next);
   uint32_t cn = gap;                    // byte 0: bits consumed; bits 8 and up: codes counted
   while ((cn & 0xffu) <= 64u - (uint32_t)kK) {
     uint32_t meta = lds_load<uint32_t>(t.dec + dec_offset(w) + 4u);
-    if (meta == 0u) {
-      uint32_t s, n;
-      walk_from(l, lds_load<uint32_t>(t.dec + dec_offset(w)), top_bits(w, next, cn & 0xffu), s, n);
-      meta = n | 0x100u;
+    if (meta & kUnsettled) {
+      meta = entry_meta(walk_from(l, lds_load<uint32_t>(t.dec + dec_offset(w)), meta, top_bits(w, next31, cn & 0xffu)));
       DF11_KEEP_BRANCH();
     }
     w <<= (meta & 63u);
@@ -354,10 +367,10 @@ DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo
     }
     const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
     uint32_t syms = e.x, meta = e.y;
-    if (meta == 0u) {
-      uint32_t n;
-      walk_from(l, syms, (uint32_t)(w >> 32), syms, n);   // at least 32 valid bits: c < 32, or already appended
-      meta = n | 0x100u;
+    if (meta & kUnsettled) {
+      const uint32_t long_code = walk_from(l, syms, meta, (uint32_t)(w >> 32));   // at least 32 valid bits: c < 32, or already appended
+      syms = entry_symbol(long_code);
+      meta = entry_meta(long_code);
       DF11_KEEP_BRANCH();
     }
     store32(p, syms);
@@ -376,10 +389,10 @@ DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo
       }
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
-      if (meta == 0u) {
-        uint32_t n;
-        walk_from(l, syms, (uint32_t)(w >> 32), syms, n);
-        meta = n | 0x100u;
+      if (meta & kUnsettled) {
+        const uint32_t long_code = walk_from(l, syms, meta, (uint32_t)(w >> 32));
+        syms = entry_symbol(long_code);
+        meta = entry_meta(long_code);
       }
       acc |= syms << got;
       got += 8u * (meta >> 8);
@@ -417,6 +430,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
                                     uint32_t next, uint32_t gap) {
   ChunkSyms r;
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
+  const uint64_t next31 = look_ahead(next);
   uint32_t c = gap, n = 0;
   r.ends[0] = r.ends[1] = 0;
 #pragma unroll
@@ -425,10 +439,10 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
     if (c <= 64u - (uint32_t)kK) {          // the lookup stays inside the chunk
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
-      if (meta == 0u) {
-        uint32_t len;
-        walk_from(l, syms, top_bits(w, next, c), syms, len);
-        meta = len | 0x100u;
+      if (meta & kUnsettled) {
+        const uint32_t long_code = walk_from(l, syms, meta, top_bits(w, next31, c));
+        syms = entry_symbol(long_code);
+        meta = entry_meta(long_code);
         DF11_KEEP_BRANCH();
       }
       r.syms[i] = syms;
@@ -450,10 +464,10 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
     if (todo) {
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
-      if (meta == 0u) {
-        uint32_t len;
-        walk_from(l, syms, (uint32_t)(w >> 32), syms, len);
-        meta = len | 0x100u;
+      if (meta & kUnsettled) {
+        const uint32_t long_code = walk_from(l, syms, meta, (uint32_t)(w >> 32));
+        syms = entry_symbol(long_code);
+        meta = entry_meta(long_code);
       }
       r.syms[kMainSlots + i] = syms;
       const uint32_t k = meta >> 8;

@@ -221,9 +221,10 @@ def _check_fused_rows(luts, codec=None):
     want = (d | (length << 8) | (flag.astype(np.uint32) << 15)).astype(np.uint16)
     assert np.array_equal(_host_fused_rows(luts), want)
     dec, _ = _host_tables(luts)
-    unresolved = np.nonzero(dec[:, 1] == 0)[0]
-    rows, shifts = (dec[unresolved, 0] & 0xFFFF) // 512, dec[unresolved, 0] >> 16
-    assert ((dec[unresolved, 0] & 0xFFFF) % 512 == 0).all()
+    unresolved = np.nonzero(dec[:, 1] >> 31)[0]
+    assert ((dec[:, 1] >> 31 == 1) | ((dec[:, 1] >> 8) - 1 < 4)).all()      # marked, or one to four codes
+    rows, shifts = dec[unresolved, 0] // 512, dec[unresolved, 1] & 0x7FFFFFFF
+    assert (dec[unresolved, 0] % 512 == 0).all()
     assert (rows < n_rows).all() and np.isin(shifts, (24, 16, 8, 0)).all()
     levels = (24 - shifts) // 8
     if codec is None:
@@ -286,6 +287,8 @@ def _check_tables_against_code(codec, luts):
             syms.append(r[1])
             pos += r[2]
         word, meta = int(dec[idx, 0]), int(dec[idx, 1])
+        if meta >> 31:                                    # settles no code: the words say where the lookup starts
+            meta = 0
         k, nbits = meta >> 8, meta & 0xFF
         got = [(word >> (8 * i)) & 0xFF for i in range(k)]
         assert got[: len(syms)] == syms, (idx, got, syms)
