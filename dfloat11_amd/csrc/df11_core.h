@@ -420,11 +420,10 @@ constexpr int kSlots = kMainSlots + kTailSlots;
 
 struct ChunkSyms {
   uint32_t syms[kSlots];   // symbol bytes of lookup i, first code in byte 0, unused bytes zero
-  uint32_t ends[2];        // one byte per lookup 0..7: symbols of the chunk up to and including it
+  uint32_t ends[kSlots - 1];   // symbols of the chunk up to and including lookup i
   uint32_t count;          // codes that start in the chunk
   bool overflow;           // ran out of slots: count and syms are incomplete
 };
-static_assert(kSlots <= 9, "ends holds the running count after lookups 0..7");
 
 DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
                                     uint32_t next, uint32_t gap) {
@@ -432,7 +431,6 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   const uint64_t next31 = look_ahead(next);
   uint32_t c = gap, n = 0;
-  r.ends[0] = r.ends[1] = 0;
 #pragma unroll
   for (int i = 0; i < kMainSlots; ++i) {
     r.syms[i] = 0;
@@ -450,7 +448,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
       w <<= (meta & 63u);
       c += meta & 0xffu;
     }
-    r.ends[i >> 2] |= n << (8 * (i & 3));   // also for a lane that skipped the lookup: later ones start here
+    r.ends[i] = n;                            // also for a lane that skipped the lookup: later ones start here
   }
   r.overflow = c <= 64u - (uint32_t)kK;
   uint32_t todo = 0;                          // codes that still start before the chunk ends
@@ -476,7 +474,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
       todo -= take;
       w <<= (meta & 63u);
     }
-    if (kMainSlots + i < 8) r.ends[(kMainSlots + i) >> 2] |= n << (8 * ((kMainSlots + i) & 3));
+    if (kMainSlots + i < kSlots - 1) r.ends[kMainSlots + i] = n;
   }
   r.overflow = r.overflow || todo != 0u;
   r.count = n;
@@ -497,20 +495,33 @@ DF11_HD void or32_aligned(LdsBytes p, uint32_t v) {
 #endif
 }
 
+// The 32-bit word that starts `bytes & 3` bytes into the 8-byte value {hi, lo}.
+DF11_HD uint32_t align_bytes(uint32_t hi, uint32_t lo, uint32_t bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_alignbyte(hi, lo, bytes);        // the instruction reads two bits of `bytes`
+#else
+  return (uint32_t)((((uint64_t)hi << 32) | lo) >> (8u * (bytes & 3u)));
+#endif
+}
+
 // OR the chunk's symbols into stage[at .. at + r.count), which must hold zeros
-// (`stage` is 4-byte aligned).  Each lookup's four symbol bytes go out as two
-// aligned words, shifted to their byte position; the unused bytes of a lookup
+// (`stage` is 4-byte aligned, at >= 4).  Each lookup's four symbol bytes go out as
+// two aligned words, shifted to their byte position; the unused bytes of a lookup
 // are zero and leave their neighbours alone, so no lookup needs trimming and the
 // lanes of a wavefront may write the bytes of one word in any order.
+// The two words are those at and after (pos - 1) & ~3, so that the shift is
+// (-pos) & 3 bytes to the right of {symbols, 0}, which one instruction per word
+// does from -pos itself; a lookup that starts on a word boundary ORs zero into the
+// word before it.
 DF11_HD void replay_chunk(const ChunkSyms& r, LdsBytes stage, uint32_t at) {
+  const uint32_t minus_at = 0u - at;
 #pragma unroll
   for (int i = 0; i < kSlots; ++i) {
     // lookup i starts where the lookups before it end
-    const uint32_t pos = i == 0 ? at : at + ((r.ends[(i - 1) >> 2] >> (8 * ((i - 1) & 3))) & 0xffu);
-    const uint64_t v = (uint64_t)r.syms[i] << ((pos & 3u) * 8u);
-    LdsBytes w = stage + (pos & ~3u);
-    or32_aligned(w, (uint32_t)v);
-    or32_aligned(w + 4, (uint32_t)(v >> 32));
+    const uint32_t minus_pos = i == 0 ? minus_at : minus_at - r.ends[i - 1];
+    LdsBytes w = stage + (~minus_pos & ~3u);               // (pos - 1) & ~3
+    or32_aligned(w, align_bytes(r.syms[i], 0u, minus_pos));
+    or32_aligned(w + 4, align_bytes(0u, r.syms[i], minus_pos));
   }
 }
 

@@ -119,8 +119,12 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   df11_emul_prepare(luts, codes_p, c_pos.p, c_gaps.p, n_luts, n_bytes, n_elements, ws.p);
   Exact<uint8_t> blob((size_t)tables_bytes(n_rows));   // what a workgroup copies into LDS
   memcpy(blob.p, ws.p + kWsTablesOffset, (size_t)tables_bytes(n_rows));
-  Exact<uint8_t> stage((size_t)stage_cap);
-  memset(stage.p, 0, (size_t)stage_cap);   // the kernel clears each wavefront's area once at start
+  // The staging area follows other data in the kernel's LDS (tables, other
+  // wavefronts' areas): the replay may OR zero into the word before it.
+  constexpr int kLeadIn = 16;
+  Exact<uint8_t> stage_mem((size_t)kLeadIn + (size_t)stage_cap);
+  memset(stage_mem.p, 0, (size_t)kLeadIn + (size_t)stage_cap);   // the kernel clears each wavefront's area once at start
+  struct { uint8_t* p; } stage{stage_mem.p + kLeadIn};
 
   const Tables t{blob.p + kDecOffset, blob.p + kCntTailOffset};
   const Rows l{blob.p + kRowsOffset};
@@ -163,7 +167,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
         replay = replay && thread_quota(excl[lane], count[lane], p.n_out) == count[lane];
       // Replay ORs into the staging area: it must be all zero here, which is the
       // previous sub-block's clear of stage_used() bytes and nothing else.
-      for (int i = 0; i < stage_cap; ++i)
+      for (int i = -kLeadIn; i < stage_cap; ++i)
         if (stage.p[i]) return 8;
       // Lanes run concurrently on the device, so no lane may rely on a later lane
       // repairing what it wrote.  Even sub-blocks write in ascending lane order,
@@ -174,7 +178,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
         const uint32_t quota = thread_quota(excl[lane], count[lane], p.n_out);
         // a lane with nothing to write may hold an out-of-range pointer; it must not use it
         uint8_t* dst = quota ? stage.p + p.phase + excl[lane] : nullptr;
-        if (replay) replay_chunk(regs[lane], stage.p, p.phase + excl[lane]);
+        if (replay) replay_chunk(regs[lane], stage_mem.p, (uint32_t)kLeadIn + p.phase + excl[lane]);
         else emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota, dst);
       }
       const SubSpans sp = spans_of(p);
