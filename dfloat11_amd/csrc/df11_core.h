@@ -305,20 +305,14 @@ DF11_HD void store16(LdsBytes p, uint32_t v) {
 #define DF11_KEEP_BRANCH() ((void)0)
 #endif
 
-// The window with the 32 look-ahead bits appended below its 64 - c valid bits.
-DF11_HD uint64_t with_next(uint64_t w, uint32_t next, uint32_t c) {
-  if (c == 0) return w;
-  return w | (c >= 32u ? (uint64_t)next << (c - 32u) : (uint64_t)next >> (32u - c));
-}
-
 // The next 32 stream bits at the top of window `w`, of which the 64 - c topmost
 // bits are valid chunk bits and the rest zero (c < 64); `next31` holds the 32 bits
 // that follow the chunk, shifted left by 31 (look_ahead): moved down by 63 - c
 // they line up with the window's first invalid bit.
 DF11_HD uint64_t look_ahead(uint32_t next) { return (uint64_t)next << 31; }
-DF11_HD uint32_t top_bits(uint64_t w, uint64_t next31, uint32_t c) {
-  return (uint32_t)((w | (next31 >> (63u - c))) >> 32);
-}
+// The window with the look-ahead bits appended below its 64 - c valid bits.
+DF11_HD uint64_t with_next(uint64_t w, uint64_t next31, uint32_t c) { return w | (next31 >> (63u - c)); }
+DF11_HD uint32_t top_bits(uint64_t w, uint64_t next31, uint32_t c) { return (uint32_t)(with_next(w, next31, c) >> 32); }
 
 // Byte offset of the table entry for the top kK bits of the window.
 DF11_HD uint32_t dec_offset(uint64_t w) { return ((uint32_t)(w >> 32) >> (32 - kK - 3)) & (uint32_t)((kTableEntries - 1) * 8); }
@@ -454,7 +448,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
   uint32_t todo = 0;                          // codes that still start before the chunk ends
   if (!r.overflow && c < 64u) {
     todo = t.cntt[(1u << (64u - c)) | (uint32_t)(w >> c)];
-    w = with_next(w, next, c);
+    w = with_next(w, next31, c);
   }
 #pragma unroll
   for (int i = 0; i < kTailSlots; ++i) {
