@@ -1,4 +1,6 @@
 """Seeded BF16 test tensors (as uint16 words) and the product compression pipeline."""
+import os
+
 import numpy as np
 import torch
 
@@ -204,3 +206,13 @@ def short_positions_case(oracle, seed, n_full_blocks):
     assert n_blocks == n_full_blocks + 1 and pos.size == n_blocks and int(pos[-1]) == e.size
     w = oracle.merge_bf16(e, sm)
     return w, dict(luts=luts, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps)
+
+
+def locked_make(directory, *targets):
+    """`make` in `directory`, one process at a time: test workers that run in parallel
+    would otherwise build the same out-of-date target at once and load half-written files."""
+    import fcntl
+    import subprocess
+    with open(os.path.join(directory, ".make.lock"), "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        subprocess.run(["make", "-s", "-C", directory, *targets], check=True)

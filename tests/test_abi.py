@@ -3,6 +3,7 @@ import os
 import re
 
 from dfloat11_amd import _native, build
+from tests.df11_cases import locked_make
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -67,7 +68,7 @@ def test_plain_c_caller_builds_against_the_header():
     libraries are usable without a HIP compiler, Python or torch."""
     import subprocess
     d = os.path.join(ROOT, "tests", "abi")
-    subprocess.run(["make", "-s", "-C", d], check=True)
+    locked_make(d)
     out = subprocess.run(["ldd", os.path.join(d, "abi_roundtrip")], capture_output=True, text=True, check=True).stdout
     assert "libdf11_hip.so" in out and "libdf11_codec.so" in out and "not found" not in out
 

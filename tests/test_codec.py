@@ -4,7 +4,7 @@ import pytest
 
 from dfloat11_amd import dfloat11_utils as U
 from oracle.df11_oracle import EOF
-from tests.df11_cases import KINDS, compress_product, make_case
+from tests.df11_cases import locked_make, KINDS, compress_product, make_case
 
 
 def _oracle_table(codec):
@@ -268,7 +268,7 @@ def test_codec_under_sanitizers():
     import os
     import subprocess
     d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
-    subprocess.run(["make", "-s", "-C", d, "df11_codec_san"], check=True)
+    locked_make(d, "df11_codec_san")
     res = subprocess.run([os.path.join(d, "df11_codec_san"), "60"], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, (res.stdout + res.stderr)[-3000:]
     assert "0 failures" in res.stdout and "32 bits" in res.stdout

@@ -9,7 +9,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from tests.df11_cases import (KINDS, compress_product, make_case, max_elems_per_block,
+from tests.df11_cases import (locked_make, KINDS, compress_product, make_case, max_elems_per_block,
                               random_code_case)
 
 EMUL_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
@@ -17,7 +17,7 @@ EMUL_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
 
 @pytest.fixture(scope="module")
 def emul():
-    subprocess.run(["make", "-s", "-C", EMUL_DIR], check=True)
+    locked_make(EMUL_DIR)
     L = ctypes.CDLL(os.path.join(EMUL_DIR, "libdf11_emul.so"))
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     L.df11_emul_decode.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, i32, i32, i32]

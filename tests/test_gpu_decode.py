@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from dfloat11_amd import decode as D
-from tests.df11_cases import KINDS, compress_product, make_case, random_code_case, short_positions_case
+from tests.df11_cases import locked_make, KINDS, compress_product, make_case, random_code_case, short_positions_case
 
 pytestmark = pytest.mark.gpu
 
@@ -145,7 +145,7 @@ def test_gpu_workspace_matches_host_build():
     emul_dir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
     lib_path = os.path.join(emul_dir, "libdf11_emul.so")
     if not os.path.exists(lib_path):
-        subprocess.run(["make", "-s", "-C", emul_dir, "libdf11_emul.so"], check=True)
+        locked_make(emul_dir, "libdf11_emul.so")
     L = ctypes.CDLL(lib_path)
     vp = ctypes.c_void_p
     L.df11_emul_prepare.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, vp]
@@ -387,7 +387,7 @@ def test_gpu_plain_c_caller_round_trip(n):
     print(f"case plain C caller n={n}", flush=True)
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "abi", "abi_roundtrip")
     if not os.path.exists(exe):
-        subprocess.run(["make", "-s", "-C", os.path.dirname(exe)], check=True)
+        locked_make(os.path.dirname(exe))
     res = subprocess.run([exe, str(n)], capture_output=True, text=True, timeout=100)
     assert res.returncode == 0, res.stdout + res.stderr
     assert "mismatches 0" in res.stdout
