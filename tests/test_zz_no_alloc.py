@@ -81,3 +81,31 @@ def test_static_workspace_rejects_streams_beyond_its_capacity():
     assert lib.df11_error_string(rc) == b"buffer too small or fixed capacity exceeded"
     assert lib.df11_decode_static_workspace(p, p, p, p, p, p, 2, 0, 0, 0, None) == 0     # empty stream
     assert lib.df11_decode_static_workspace(None, p, p, p, p, p, 2, 8, 1, 0, None) == -1
+
+
+def test_static_workspace_decode_in_a_captured_graph():
+    """The callers this entry point is for include code under graph capture: captured,
+    every replay rebuilds the tables in the library's array and reproduces the eager
+    result, also after an eager call for another stream has overwritten that array."""
+    lib = _native.hip_lib()
+    w = make_case("laplace", 900_001, 23)
+    other = make_case("fib", 50_000, 29)
+    g, g_other = _upload(compress_product(w)), _upload(compress_product(other))
+    out = torch.zeros(w.size, dtype=torch.bfloat16, device=DEV)
+    out_other = torch.zeros(other.size, dtype=torch.bfloat16, device=DEV)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        assert _decode_static(lib, g, w.size, out, 0) == 0      # first use outside the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert _decode_static(lib, g, w.size, out, 0) == 0
+    for replay in range(3):
+        print(f"case static workspace graph replay {replay}", flush=True)
+        out.fill_(1.0)
+        assert _decode_static(lib, g_other, other.size, out_other, 0) == 0   # eager, same shared array
+        torch.cuda.synchronize()
+        assert np.array_equal(out_other.view(torch.int16).cpu().numpy().view(np.uint16), other)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), w)
