@@ -64,7 +64,7 @@ def cpu_baseline(stream, original_u16, budget_s=12.0):
     # whole stream if it fits the budget of CPU work, else a prefix of it; repeated so
     # that about `budget_s` core-seconds are spent, and the median pass is reported
     sample = int(min(n_blocks, max(n_threads, budget_s / per_block_1t)))
-    repeats = int(max(1, min(7, budget_s / (sample * per_block_1t))))
+    repeats = int(max(1, min(15, budget_s / (sample * per_block_1t))))
     bounds = [sample * i // n_threads for i in range(n_threads + 1)]
     times = []
     for _ in range(repeats):
