@@ -231,7 +231,6 @@ struct DecodeSizes {
   int32_t stage_cap;      // bytes of staging per wavefront, multiple of 16
   int32_t codes_aligned;  // codes pointer is 8-byte aligned
   int32_t vec_ok;         // sign_mantissa 8-byte aligned and out 16-byte aligned
-  int32_t phase_priority; // wavefront priority by phase instead of by turn (see the decode loop)
 };
 
 // kPrefetch (template parameter of the decode body): body groups per lane whose
@@ -290,7 +289,7 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-template <int kPrefetchGroups, bool kStreaming>
+template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority>
 __device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
@@ -345,18 +344,19 @@ __device__ __forceinline__ void decode_body(
   // starting point given by its slot on the SIMD: over time every wavefront gets
   // the same share and all of them finish together.
   // A stream of few sub-blocks per wavefront has no long run to even out; there
-  // (z.phase_priority) the priority follows the phase instead: lowest while a
-  // wavefront decodes, highest while it writes out, so that stores and the next
-  // requests are issued as soon as they can be and the decodes of the other
-  // wavefronts fill the gaps.
-  const bool phase_priority = z.phase_priority != 0;   // uniform
+  // (kPhasePriority) the priority follows the phase instead: lowest while a
+  // wavefront decodes, highest while it writes out and requests the next
+  // sub-block's inputs, so that stores and loads are issued as soon as they can be
+  // and the decodes of the other wavefronts fill the gaps.
   uint32_t turn = __builtin_amdgcn_s_getreg((3 << 11) | 4);   // HW_ID.WAVE_ID, the slot on the SIMD
   for (; sub < z.n_subs; sub += stride) {
-    switch (phase_priority ? 0u : (turn++ & 3u)) {   // s_setprio takes an immediate
-      case 0: __builtin_amdgcn_s_setprio(0); break;
-      case 1: __builtin_amdgcn_s_setprio(1); break;
-      case 2: __builtin_amdgcn_s_setprio(2); break;
-      default: __builtin_amdgcn_s_setprio(3); break;
+    if (!kPhasePriority) {
+      switch (turn++ & 3u) {   // s_setprio takes an immediate
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
+      }
     }
     // ---- requests whose latency the two decode passes hide: the next
     // sub-block's inputs and this one's sign|mantissa bytes
@@ -396,6 +396,7 @@ __device__ __forceinline__ void decode_body(
     if (edge_hint_ok) edge_byte = sm0[edge_hint];
 
     // ---- decode, and the exclusive offsets inside the wavefront
+    if (kPhasePriority) __builtin_amdgcn_s_setprio(0);
     const Chunk c{__builtin_bswap32(cur.d0), __builtin_bswap32(cur.d1), __builtin_bswap32(cur.d2)};
     const uint32_t gap_word = __builtin_bswap32(cur.gap_raw) >> 16;   // the two bytes, big-endian
     const uint32_t gap = (gap_word >> gap_shift) & 31u;
@@ -423,7 +424,7 @@ __device__ __forceinline__ void decode_body(
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     // ---- stream out
-    if (phase_priority) __builtin_amdgcn_s_setprio(3);
+    if (kPhasePriority) __builtin_amdgcn_s_setprio(3);
     // Vector loads and stores share one in-order completion counter on this
     // hardware, so the first use of a loaded value after a store waits for that
     // store to reach memory.  Every value requested above is therefore claimed
@@ -504,25 +505,29 @@ __device__ __forceinline__ void decode_body(
 //   deepest  2 workgroups per CU, 6 groups requested early, for streams of short
 //            codes (a sub-block of one-bit codes is 8 groups per lane): 74 % of the
 //            HBM peak on the all-zero mix against 68 % with `wide`.
+// The deep plans come in a second compilation (`_short`) for streams of few
+// sub-blocks per wavefront, which sets wavefront priorities by phase (see the loop).
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
-#define DF11_DECODE_KERNEL(name, prefetch, streaming, waves_per_simd)                             \
+#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd)             \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
                                                                              waves_per_simd)))    \
   void name(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,         \
             const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,                         \
             const uint8_t* __restrict__ ws, const DecodeSizes z) {                                \
-    decode_body<prefetch, streaming>(codes, sign_mantissa, gaps, out, ws, z);                     \
+    decode_body<prefetch, streaming, phase_priority>(codes, sign_mantissa, gaps, out, ws, z);     \
   }
-DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, 6)
-DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, 4)
-DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6)
+DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4)
+DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4)
+DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4)
 #undef DF11_DECODE_KERNEL
 
 typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);
 struct LaunchPlan {
   DecodeKernel kernel;
   int groups_per_cu;
-  bool streams_deep;   // one of the plans for large streams
+  DecodeKernel kernel_short;   // for up to kMaxRoundsForPhasePriority sub-blocks per wavefront, or null
 };
 constexpr int kWideGroupsPerCu = 3;
 constexpr int kDeepGroupsPerCu = 2;
@@ -539,17 +544,18 @@ std::atomic<int> g_forced_plan{-1};   // df11_force_launch_plan: -1 = choose per
 
 LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
   switch (g_forced_plan.load(std::memory_order_relaxed)) {
-    case DF11_PLAN_WIDE: return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, false};
-    case DF11_PLAN_DEEP: return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, true};
-    case DF11_PLAN_DEEPEST: return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, true};
+    case DF11_PLAN_WIDE: return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
+    case DF11_PLAN_DEEP: return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short};
+    case DF11_PLAN_DEEPEST: return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short};
     default: break;
   }
   const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
   if (n_elements < kMinElemsPerWaveForDeep * wide_waves || elems_per_sub < kMinElemsPerSubForDeep)
-    return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, false};
-  if (elems_per_sub < kMinElemsPerSubForDeepest) return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, true};
-  return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, true};
+    return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
+  if (elems_per_sub < kMinElemsPerSubForDeepest)
+    return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short};
+  return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short};
 }
 
 // Plain streaming copy, 16 bytes per lane: the known-traffic kernel against
@@ -578,7 +584,8 @@ int device_info(DeviceInfo& info) {
     if (e != hipSuccess) return hip_fail(e);
     // the decode kernels address their LDS from a constant base, which holds only
     // as long as they have no static LDS of their own
-    for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deepest}) {
+    for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deep_short, decode_kernel_deepest,
+                           decode_kernel_deepest_short}) {
       hipFuncAttributes attr;
       e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(k));
       if (e != hipSuccess) return hip_fail(e);
@@ -657,10 +664,11 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, plan.groups_per_cu);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
-  z.phase_priority = plan.streams_deep && z.n_subs <= (int64_t)kMaxRoundsForPhasePriority * grid * kWavesPerGroup;
+  const bool few_rounds = z.n_subs <= (int64_t)kMaxRoundsForPhasePriority * grid * kWavesPerGroup;
+  const DecodeKernel kernel = few_rounds && plan.kernel_short ? plan.kernel_short : plan.kernel;
 
   (void)luts;   // read by df11_prepare only: the decode finds them fused in the workspace
-  hipLaunchKernelGGL(plan.kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s,
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s,
                      encoded_exponent, sign_mantissa, gaps, outputs, ws, z);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? DF11_OK : hip_fail(e);
