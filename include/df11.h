@@ -123,7 +123,9 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
 /*
  * The decode kernel exists in three launch plans (workgroups resident per CU and
  * depth of its requests for sign_mantissa bytes); df11_decode picks one per
- * stream from its size and its elements per 512 bytes of bitstream.  This call
+ * stream from its size and its elements per 512 bytes of bitstream (and, within
+ * the two plans for large streams, how wavefront priorities are set from the
+ * stream's size, which this call leaves alone).  This call
  * pins the plan for every later decode of the process, or hands the choice back
  * (DF11_PLAN_AUTO).  Testing and measurement aid with no counterpart in the
  * reference: every plan decodes every stream to the same bits.
