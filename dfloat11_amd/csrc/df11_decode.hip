@@ -494,10 +494,10 @@ __device__ __forceinline__ void decode_body(
 // elements):
 //   wide     3 workgroups per CU (6 wavefronts per SIMD), 2 groups requested early,
 //            plain (cacheable) loads.
-//            Best when wavefronts are the scarce resource: streams of fewer than
-//            about 38 M elements (a few rounds of sub-blocks: the launch is
-//            latency-bound) and streams whose decode is bound by vector
-//            instructions (long codes, few elements per sub-block).
+//            Best when wavefronts are the scarce resource: streams whose decode is
+//            bound by vector instructions (long codes, few elements per sub-block),
+//            and those streams of fewer than about 38 M elements (a few rounds of
+//            sub-blocks: the launch is latency-bound) whose rounds fill it well.
 //   deep     2 workgroups per CU (4 per SIMD), 3 groups requested early: a typical
 //            sub-block is 3 groups per lane, so the whole write-out runs on bytes
 //            that are already there.  Fewer, deeper memory streams: 1 % (218 M
@@ -506,7 +506,10 @@ __device__ __forceinline__ void decode_body(
 //            codes (a sub-block of one-bit codes is 8 groups per lane): 74 % of the
 //            HBM peak on the all-zero mix against 68 % with `wide`.
 // The deep plans come in a second compilation (`_short`) for streams of few
-// sub-blocks per wavefront, which sets wavefront priorities by phase (see the loop).
+// sub-blocks per wavefront, which sets wavefront priorities by phase (see the loop),
+// and `deep` in a third (`_small`) that also reads with plain loads, for the streams
+// under 38 M elements that fit its rounds better than those of `wide` (a stream that
+// small may still sit in the memory-side cache).
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
 #define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd)             \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
@@ -519,6 +522,7 @@ __device__ __forceinline__ void decode_body(
 DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6)
 DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4)
 DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4)
 DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4)
 DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4)
 #undef DF11_DECODE_KERNEL
@@ -550,9 +554,21 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
     default: break;
   }
   const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
+  const int64_t deep_waves = (int64_t)cus * kDeepGroupsPerCu * kWavesPerGroup;
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
-  if (n_elements < kMinElemsPerWaveForDeep * wide_waves || elems_per_sub < kMinElemsPerSubForDeep)
-    return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
+  if (elems_per_sub < kMinElemsPerSubForDeep) return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
+  if (n_elements < kMinElemsPerWaveForDeep * wide_waves) {
+    // A few rounds of sub-blocks.  Under the wide plan such a launch takes as long as
+    // its rounds, full or not: 0.79 W + ceil(n / W) W in units of one sub-block's share
+    // of a full round of W wavefronts.  Under the deep plan it grows evenly with the
+    // stream, 1.08 W + 0.91 n (measured from 2,500 to 24,000 sub-blocks read from HBM;
+    // 0.25 W kept as margin).  Short-code streams stay wide.
+    const int64_t wide_cost = (79 * wide_waves + (n_subs + wide_waves - 1) / wide_waves * wide_waves * 100);
+    const int64_t deep_cost = 133 * wide_waves + 91 * n_subs;
+    if (elems_per_sub >= kMinElemsPerSubForDeepest || (n_subs > deep_waves && wide_cost <= deep_cost))
+      return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
+    return LaunchPlan{decode_kernel_deep_small, kDeepGroupsPerCu, decode_kernel_deep_small};
+  }
   if (elems_per_sub < kMinElemsPerSubForDeepest)
     return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short};
   return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short};
@@ -584,8 +600,8 @@ int device_info(DeviceInfo& info) {
     if (e != hipSuccess) return hip_fail(e);
     // the decode kernels address their LDS from a constant base, which holds only
     // as long as they have no static LDS of their own
-    for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deep_short, decode_kernel_deepest,
-                           decode_kernel_deepest_short}) {
+    for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deep_short, decode_kernel_deep_small,
+                           decode_kernel_deepest, decode_kernel_deepest_short}) {
       hipFuncAttributes attr;
       e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(k));
       if (e != hipSuccess) return hip_fail(e);
