@@ -532,6 +532,8 @@ struct LaunchPlan {
   DecodeKernel kernel;
   int groups_per_cu;
   DecodeKernel kernel_short;   // for up to kMaxRoundsForPhasePriority sub-blocks per wavefront, or null
+  const char* name;
+  const char* name_short;
 };
 constexpr int kWideGroupsPerCu = 3;
 constexpr int kDeepGroupsPerCu = 2;
@@ -546,17 +548,24 @@ constexpr int kMaxRoundsForPhasePriority = 16;
 
 std::atomic<int> g_forced_plan{-1};   // df11_force_launch_plan: -1 = choose per stream
 
+const LaunchPlan kWide{decode_kernel_wide, kWideGroupsPerCu, nullptr, "wide", nullptr};
+const LaunchPlan kDeep{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short, "deep", "deep/short"};
+const LaunchPlan kDeepSmall{decode_kernel_deep_small, kDeepGroupsPerCu, decode_kernel_deep_small, "deep/small",
+                            "deep/small"};
+const LaunchPlan kDeepest{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short, "deepest",
+                          "deepest/short"};
+
 LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
   switch (g_forced_plan.load(std::memory_order_relaxed)) {
-    case DF11_PLAN_WIDE: return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
-    case DF11_PLAN_DEEP: return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short};
-    case DF11_PLAN_DEEPEST: return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short};
+    case DF11_PLAN_WIDE: return kWide;
+    case DF11_PLAN_DEEP: return kDeep;
+    case DF11_PLAN_DEEPEST: return kDeepest;
     default: break;
   }
   const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
   const int64_t deep_waves = (int64_t)cus * kDeepGroupsPerCu * kWavesPerGroup;
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
-  if (elems_per_sub < kMinElemsPerSubForDeep) return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
+  if (elems_per_sub < kMinElemsPerSubForDeep) return kWide;
   if (n_elements < kMinElemsPerWaveForDeep * wide_waves) {
     // A few rounds of sub-blocks.  Under the wide plan such a launch takes as long as
     // its rounds, full or not: 0.79 W + ceil(n / W) W in units of one sub-block's share
@@ -566,12 +575,15 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
     const int64_t wide_cost = (79 * wide_waves + (n_subs + wide_waves - 1) / wide_waves * wide_waves * 100);
     const int64_t deep_cost = 133 * wide_waves + 91 * n_subs;
     if (elems_per_sub >= kMinElemsPerSubForDeepest || (n_subs > deep_waves && wide_cost <= deep_cost))
-      return LaunchPlan{decode_kernel_wide, kWideGroupsPerCu, nullptr};
-    return LaunchPlan{decode_kernel_deep_small, kDeepGroupsPerCu, decode_kernel_deep_small};
+      return kWide;
+    return kDeepSmall;
   }
-  if (elems_per_sub < kMinElemsPerSubForDeepest)
-    return LaunchPlan{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short};
-  return LaunchPlan{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short};
+  if (elems_per_sub < kMinElemsPerSubForDeepest) return kDeep;
+  return kDeepest;
+}
+
+bool few_rounds(int64_t n_subs, int64_t grid) {
+  return n_subs <= (int64_t)kMaxRoundsForPhasePriority * grid * kWavesPerGroup;
 }
 
 // Plain streaming copy, 16 bytes per lane: the known-traffic kernel against
@@ -680,8 +692,7 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, plan.groups_per_cu);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
-  const bool few_rounds = z.n_subs <= (int64_t)kMaxRoundsForPhasePriority * grid * kWavesPerGroup;
-  const DecodeKernel kernel = few_rounds && plan.kernel_short ? plan.kernel_short : plan.kernel;
+  const DecodeKernel kernel = few_rounds(z.n_subs, grid) && plan.kernel_short ? plan.kernel_short : plan.kernel;
 
   (void)luts;   // read by df11_prepare only: the decode finds them fused in the workspace
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), lds_bytes, s,
@@ -779,6 +790,16 @@ int df11_force_launch_plan(int plan) {
   if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_DEEPEST) return DF11_ERR_INVALID_ARGUMENT;
   g_forced_plan.store(plan, std::memory_order_relaxed);
   return DF11_OK;
+}
+
+const char* df11_launch_plan_name(int64_t n_bytes, int64_t n_elements, int32_t compute_units) {
+  if (n_bytes <= 0 || n_elements <= 0 || compute_units <= 0) return "";
+  const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
+  const LaunchPlan plan = plan_launch(n_subs, n_elements, compute_units);
+  int64_t grid = (int64_t)compute_units * plan.groups_per_cu;
+  const int64_t needed = (n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
+  if (grid > needed) grid = needed;
+  return few_rounds(n_subs, grid) && plan.kernel_short ? plan.name_short : plan.name;
 }
 
 int df11_calibration_copy(const void* src, void* dst, int64_t n_bytes, void* stream) {

@@ -137,6 +137,16 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
 int df11_force_launch_plan(int plan);
 
 /*
+ * Which compilation of the decode kernel df11_decode launches for a stream of
+ * n_bytes of encoded_exponent and n_elements on a device of compute_units CUs
+ * (when the LDS the stream needs leaves room for the plan's workgroups per CU):
+ * "wide", "deep", "deep/short", "deep/small", "deepest" or "deepest/short";
+ * "" for sizes that are not positive.  Needs no GPU.  Testing aid with no
+ * counterpart in the reference.
+ */
+const char *df11_launch_plan_name(int64_t n_bytes, int64_t n_elements, int32_t compute_units);
+
+/*
  * Streaming device copy of n_bytes (multiple of 16, both pointers 16-byte
  * aligned).  Measurement aid with no counterpart in the reference: a kernel of
  * known HBM traffic against which profiler byte counters are calibrated.

@@ -78,3 +78,37 @@ def test_launch_plan_override_is_validated():
     assert hip.df11_force_launch_plan(3) == -1 and hip.df11_force_launch_plan(-2) == -1
     for plan in (0, 1, 2, -1):
         assert hip.df11_force_launch_plan(plan) == 0
+
+
+def test_launch_plan_follows_stream_size_and_code_lengths():
+    """The choice among the compilations of the decode kernel, asked without a GPU for a
+    device of 256 CUs: streams of N(0, 0.02) weights (0.324 bitstream bytes per element),
+    of one-bit codes (1/8) and of incompressible exponents (1.16)."""
+    hip = _native.hip_lib()
+
+    def plan(n_elements, bytes_per_element=0.324, cus=256):
+        return hip.df11_launch_plan_name(int(n_elements * bytes_per_element), int(n_elements), cus).decode()
+
+    assert plan(218_103_808) == "deep"                 # a Llama-3-8B decoder block
+    assert plan(622_329_856) == "deep"                 # a 151936 x 4096 embedding
+    assert plan(4096 * 14336) == "deep/short"          # few sub-blocks per wavefront: priorities by phase
+    assert plan(100_000_000) == "deep/short"
+    assert plan(120_000_000) == "deep"
+    assert plan(4096 * 4096) == "wide"                 # 1.7 rounds of the wide plan, 2.6 of the deep one
+    assert plan(8_000_000) == "wide"
+    assert plan(20_000_000) == "deep/small"            # 2.1 rounds of the wide plan
+    assert plan(30_000_000) == "deep/small"
+    assert plan(100_000) == "deep/small"               # a single round either way
+    assert plan(622_329_856, 0.125) == "deepest"       # one-bit codes
+    assert plan(4096 * 14336, 0.125) == "deepest/short"
+    assert plan(4096 * 4096, 0.125) == "wide"
+    for n in (1000, 4096 * 4096, 4096 * 14336, 622_329_856):
+        assert plan(n, 1.16) == "wide"                 # decode-bound whatever the size
+    assert plan(4096 * 14336, cus=64) == "deep"        # the same matrix is 36 rounds on a quarter of the CUs
+    assert hip.df11_launch_plan_name(0, 10, 256) == b"" and hip.df11_launch_plan_name(10, 10, 0) == b""
+    # a pinned plan answers for itself
+    assert hip.df11_force_launch_plan(0) == 0
+    try:
+        assert plan(218_103_808) == "wide"
+    finally:
+        assert hip.df11_force_launch_plan(-1) == 0
