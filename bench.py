@@ -307,7 +307,10 @@ def main():
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": profiled_traffic(),
-                     "kernel": "decode_kernel_deep", "avg_launch_ms": avg_kernel_ms},
+                     "kernel": "decode_kernel_" + lib.df11_launch_plan_name(
+                         int(n_bytes), int(n_elements),
+                         torch.cuda.get_device_properties(dev).multi_processor_count).decode().replace("/", "_"),
+                     "avg_launch_ms": avg_kernel_ms},
     }
     if not a.no_mixes:
         copies.clear()
