@@ -20,8 +20,9 @@
 //   5. streams the staging area out: 8 exponent bytes (LDS) + 8 sign|mantissa
 //      bytes -> one 16-byte BF16 store per lane, contiguous across the wavefront,
 //      in batches of 64 lanes that start on 256-byte lines of the output.
-// The kernel is bound by HBM; the decode (about 70 % of the memory time) is
-// hidden under it with three workgroups per CU.
+// The kernel is bound by HBM; the decode (vector instructions for a little over
+// half of the memory time on weight-like streams) is hidden under it with two or
+// three workgroups per CU (the launch plans further down).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
