@@ -174,6 +174,47 @@ def random_code_case(seed, max_n=20_000):
     return w, cases
 
 
+def max_rows_case(seed, n):
+    """(w, streams per fill policy) for a hand-made code that needs every LUT row the
+    layout has: the root, thirteen second-level rows (first bytes 0xF0..0xFC, 9-bit
+    codes), and a chain below first byte 0xFD through a second-, a third- and a
+    fourth-level row (17-, 25- and 32-bit codes, the longest for exponents >= 240):
+    16 sub-tables, luts of 18 rows.  Exponents are drawn so that long codes are common."""
+    rng = np.random.default_rng(seed)
+    codes = [(1, 0b0), (2, 0b10), (3, 0b110), (4, 0b1110), (8, 0xFE), (8, 0xFF)]
+    for first in range(0xF0, 0xFD):
+        codes += [(9, first << 1), (9, (first << 1) | 1)]
+    codes += [(9, 0xFD << 1)]                                   # 0xFD 0
+    codes += [(17, (0xFDFF << 1))]                              # 0xFD 0xFF 0
+    long_codes = [(25, 0xFDFFFF << 1), (32, 0xFDFFFFFE), (30, (0xFDFFFF << 6) | 0b100000)]
+    eof = (32, 0xFDFFFFFF)
+    code_len = np.zeros(256, np.uint8)
+    code_val = np.zeros(256, np.uint32)
+    low = list(rng.permutation(240))
+    high = list(rng.permutation(np.arange(240, 256)))
+    for l, v in codes:
+        s = low.pop()
+        code_len[s], code_val[s] = l, v
+    for l, v in long_codes:
+        s = high.pop()
+        code_len[s], code_val[s] = l, v
+    codec = U.DF11Codec(code_len, code_val, eof[0], eof[1])
+    luts = U.get_luts(codec.get_code_table()).numpy()
+    assert luts.shape[0] == 18, luts.shape
+    syms = np.array([s for s in range(256) if code_len[s]], dtype=np.uint8)
+    p = 1.0 / np.sqrt(code_len[syms].astype(np.float64))        # long codes nearly as likely as short ones
+    e = rng.choice(syms, n, p=p / p.sum())
+    enc, gaps, pos = U.encode(e, codec)
+    sm = rng.integers(0, 256, n).astype(np.uint8)
+    w = (((sm.astype(np.uint16) & 0x80) << 8) | (e.astype(np.uint16) << 7) | (sm & 0x7F)).astype(np.uint16)
+    cases = {}
+    for policy in ("product", "forward", "random"):
+        l = luts if policy == "product" else refill_unowned_slots(luts, codec, policy, rng)
+        cases[policy] = dict(luts=l, encoded_exponent=enc, sign_mantissa=sm, output_positions=pos, gaps=gaps,
+                             codec=codec)
+    return w, cases
+
+
 def short_positions_case(oracle, seed, n_full_blocks):
     """A stream laid out by the oracle's restatement of the reference encoder whose
     output_positions comes out one entry short: the last code starts in block

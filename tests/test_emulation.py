@@ -9,7 +9,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from tests.df11_cases import (locked_make, KINDS, compress_product, make_case, max_elems_per_block,
+from tests.df11_cases import (locked_make, KINDS, compress_product, make_case, max_elems_per_block, max_rows_case,
                               random_code_case)
 
 EMUL_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emul")
@@ -362,6 +362,22 @@ def test_emulated_kernel_random_codes_and_fillings(emul, oracle, chunk):
                 assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (seed, policy, two_pass)
             ran += 1
     assert ran > 20
+
+
+@pytest.mark.parametrize("n", [1, 700, 40_000])
+def test_emulated_kernel_every_lut_row(emul, oracle, n):
+    """A code that fills the layout's 16 sub-tables on all four levels (luts of 18 rows,
+    codes of 1 to 32 bits) x three fillings of the unowned slots: derived tables from
+    their definition, and kernel == oracle == original words on both decode routes."""
+    w, cases = max_rows_case(300 + n, n)
+    for policy, c in cases.items():
+        _check_tables_against_code(c["codec"], c["luts"])
+        assert _check_fused_rows(c["luts"], c["codec"]) > 0
+        ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                              c["output_positions"], c["gaps"])
+        assert np.array_equal(ref, w), policy
+        for two_pass in (False, True):
+            assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (policy, two_pass)
 
 
 def test_emulated_kernel_few_elements_many_symbols(emul, oracle):

@@ -8,7 +8,8 @@ import pytest
 import torch
 
 from dfloat11_amd import decode as D
-from tests.df11_cases import locked_make, KINDS, compress_product, make_case, random_code_case, short_positions_case
+from tests.df11_cases import (locked_make, KINDS, compress_product, make_case, max_rows_case, random_code_case,
+                              short_positions_case)
 
 pytestmark = pytest.mark.gpu
 
@@ -129,6 +130,19 @@ def test_gpu_random_codes_and_fillings(oracle):
         sm = rng.integers(0, 256, n).astype(np.uint16)
         w = (((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)).astype(np.uint16)
         assert np.array_equal(gpu_decode(compress_product(w)), w)
+
+
+@pytest.mark.parametrize("n", [1, 700, 40_000, 2_000_000])
+def test_gpu_every_lut_row(oracle, n):
+    """A code that fills the layout's 16 sub-tables on all four levels (luts of 18 rows,
+    codes of 1 to 32 bits, long codes common) x three fillings of the unowned slots."""
+    w, cases = max_rows_case(300 + n, n)
+    for policy, c in cases.items():
+        print(f"case every LUT row n={n} filling={policy}", flush=True)
+        ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
+                              c["output_positions"], c["gaps"])
+        assert np.array_equal(ref, w)
+        assert np.array_equal(gpu_decode(c), ref), policy
 
 
 @pytest.mark.parametrize("kind", ["normal", "zeros", "fib"])
