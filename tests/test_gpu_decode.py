@@ -143,6 +143,9 @@ def test_gpu_every_lut_row(oracle, n):
                               c["output_positions"], c["gaps"])
         assert np.array_equal(ref, w)
         assert np.array_equal(gpu_decode(c), ref), policy
+    # all 17 decode rows together with the staging of the worst case (4096 elements per
+    # 512 bytes of bitstream): the largest LDS allocation a launch can ask for
+    assert np.array_equal(gpu_decode(cases["product"], max_elems=0), w)
 
 
 @pytest.mark.parametrize("kind", ["normal", "zeros", "fib"])
