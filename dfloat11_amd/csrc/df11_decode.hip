@@ -571,10 +571,12 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
     // A few rounds of sub-blocks.  Under the wide plan such a launch takes as long as
     // its rounds, full or not: 0.79 W + ceil(n / W) W in units of one sub-block's share
     // of a full round of W wavefronts.  Under the deep plan it grows evenly with the
-    // stream, 1.08 W + 0.91 n (measured from 2,500 to 24,000 sub-blocks read from HBM;
-    // 0.25 W kept as margin).  Short-code streams stay wide.
+    // stream, 1.08 W + 0.91 n (measured from 2,500 to 24,000 sub-blocks read from HBM),
+    // within 0.25 W up to two rounds of W and proportionally closer beyond: kept as
+    // margin.  Short-code streams stay wide.
     const int64_t wide_cost = (79 * wide_waves + (n_subs + wide_waves - 1) / wide_waves * wide_waves * 100);
-    const int64_t deep_cost = 133 * wide_waves + 91 * n_subs;
+    const int64_t margin = n_subs > 2 * wide_waves ? 25 * wide_waves * 2 * wide_waves / n_subs : 25 * wide_waves;
+    const int64_t deep_cost = 108 * wide_waves + margin + 91 * n_subs;
     if (elems_per_sub >= kMinElemsPerSubForDeepest || (n_subs > deep_waves && wide_cost <= deep_cost))
       return kWide;
     return kDeepSmall;
