@@ -1,9 +1,13 @@
-"""The two remaining measurement workloads of the DF11 decode path on one MI355X
+"""The remaining measurement workloads of the DF11 decode path on one MI355X
 (bench.py holds the headline one).  One JSON line per result.
 
   --workload mixes         decode GB/s and bit-exactness per adversarial exponent
                            distribution, on a 151936x4096 embedding-shaped tensor and
                            a 4096x14336 matrix
+  --workload sizes         N(0, 0.02) tensors of 2 M to 120 M elements: which compilation
+                           of the kernel the library launches, and the time per launch
+                           with the input read from HBM (device copies decoded in turn)
+                           and from the memory-side cache (one copy over and over)
   --workload flux-offload  one forward pass of a FLUX.1-dev-shaped block stack (hidden
                            3072, 19 double-stream + 38 single-stream blocks) whose
                            compressed streams live in pinned host memory and are copied
@@ -120,6 +124,86 @@ def time_decode(torch, w, steps, warmup, preheat_ms=150.0):
         "compressed_over_bf16": (enc.numel() + n + gaps.numel() + 4 * pos.numel()) / (2.0 * n),
         "max_elems_per_subblock": int(max_sub), "encode_seconds_host": t_encode,
     }
+
+
+SIZES_M = (2, 4, 6, 8, 10, 12, 14, 16.777216, 20, 23, 25, 28, 30, 34, 37, 38, 45, 58.720256, 80, 100, 120)
+
+
+def time_copies_in_turn(torch, w, launches=40, preheat_ms=150.0):
+    """Encode w once, keep enough device copies of the stream that a launch never finds its
+    input in the 256 MB memory-side cache (at least 600 MB of inputs in all), and decode them
+    in turn, back to back, into one output; then the first copy alone, over and over."""
+    from dfloat11_amd import _native
+    from dfloat11_amd import decode as D
+    from dfloat11_amd import dfloat11_utils as U
+    dev = w.device
+    w_cpu = w.cpu().flatten()
+    _, counter = U.get_codec(w_cpu)
+    codec, _, table = U.get_32bit_codec(counter)
+    luts = U.get_luts(table)
+    enc, sm, pos, gaps, _ = U.encode_weights([w_cpu], codec)
+    n = w_cpu.numel()
+    input_bytes = enc.numel() + sm.numel() + gaps.numel() + 4 * pos.numel()
+    n_copies = int(min(64, max(2, -(-600_000_000 // input_bytes))))
+    lib = _native.hip_lib()
+    out = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    keep, calls = [], []
+    for _ in range(n_copies):
+        d = [t.to(dev) for t in (luts, enc, sm, gaps)] + [pos.view(torch.uint8).to(dev)]
+        ws, max_sub = D.prepare(d[0], d[1], d[4], d[3], n)
+        keep.append((d, ws))
+        calls.append((d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[4].data_ptr(), d[3].data_ptr(),
+                      out.data_ptr(), int(luts.shape[0]), int(enc.numel()), int(n), ws.data_ptr(), int(max_sub),
+                      torch.cuda.current_stream(dev).cuda_stream))
+    D.decode(keep[0][0][0], keep[0][0][1], keep[0][0][2], keep[0][0][4], keep[0][0][3], out, keep[0][1], calls[0][10])
+    torch.cuda.synchronize()
+    bit_exact = bool(torch.equal(out.view(torch.int16), w.flatten().view(torch.int16)))
+
+    def per_launch(which):
+        t0 = time.perf_counter()
+        i = 0
+        while (time.perf_counter() - t0) * 1e3 < preheat_ms:
+            for _ in range(16):
+                lib.df11_decode(*calls[which(i)])
+                i += 1
+            torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            b0, b1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            b0.record()
+            for _ in range(launches):
+                if lib.df11_decode(*calls[which(i)]) != 0:
+                    raise RuntimeError("df11_decode failed")
+                i += 1
+            b1.record()
+            torch.cuda.synchronize()
+            times.append(b0.elapsed_time(b1) / launches)
+        return float(np.median(times))
+
+    in_turn = per_launch(lambda i: i % n_copies)
+    same = per_launch(lambda i: 0)
+    algo = algorithmic_bytes(enc.numel(), n, luts.shape[0])
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    return {
+        "n_elements": n, "bitstream_sub_blocks": -(-enc.numel() // 512), "algorithmic_bytes": algo,
+        "kernel": "decode_kernel_" + lib.df11_launch_plan_name(int(enc.numel()), int(n), cus).decode().replace("/", "_"),
+        "device_copies": n_copies, "copies_in_turn_ms_per_launch": in_turn,
+        "copies_in_turn_hbm_frac": algo / (in_turn * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "same_copy_ms_per_launch": same, "same_copy_hbm_frac": algo / (same * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "bit_exact": bit_exact,
+    }
+
+
+def run_sizes(a, torch, dev):
+    ok = True
+    for m in SIZES_M:
+        w = make_mix(torch, "normal", int(m * 1e6), dev, seed=7)
+        r = time_copies_in_turn(torch, w)
+        del w
+        torch.cuda.empty_cache()
+        ok = ok and r["bit_exact"]
+        print(json.dumps({"workload": "sizes", "mix": "normal", **r}), flush=True)
+    return ok
 
 
 def run_mixes(a, torch, dev):
@@ -347,7 +431,7 @@ def run_flux(a, torch, dev):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--workload", choices=["mixes", "flux-offload"], required=True)
+    ap.add_argument("--workload", choices=["mixes", "sizes", "flux-offload"], required=True)
     ap.add_argument("--mix", choices=MIXES + ("normal",), default=None, help="mixes: only this distribution")
     ap.add_argument("--tensor", choices=[t[0] for t in ALL_SHAPES], default=None, help="mixes: only this tensor")
     ap.add_argument("--steps", type=int, default=50)
@@ -362,7 +446,7 @@ def main():
         sys.exit("bench_extra.py needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    ok = run_mixes(a, torch, dev) if a.workload == "mixes" else run_flux(a, torch, dev)
+    ok = {"mixes": run_mixes, "sizes": run_sizes, "flux-offload": run_flux}[a.workload](a, torch, dev)
     sys.exit(0 if ok else 1)
 
 

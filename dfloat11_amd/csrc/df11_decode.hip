@@ -546,6 +546,7 @@ constexpr int kMinElemsPerSubForDeepest = 2560;
 // 142 M; 0.5 % slower at 218 M, 5 % at 622 M; 9 % slower under the wide plan on a
 // decode-bound stream).
 constexpr int kMaxRoundsForPhasePriority = 16;
+constexpr int64_t kMaxInputBytesForPlainLoads = 40 << 20;   // about 30 M weight-like elements
 
 std::atomic<int> g_forced_plan{-1};   // df11_force_launch_plan: -1 = choose per stream
 
@@ -579,7 +580,10 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
     const int64_t deep_cost = 108 * wide_waves + margin + 91 * n_subs;
     if (elems_per_sub >= kMinElemsPerSubForDeepest || (n_subs > deep_waves && wide_cost <= deep_cost))
       return kWide;
-    return kDeepSmall;
+    // Plain loads pay when the stream may still be in the memory-side cache and cost 1-5 %
+    // when it comes from HBM, more the larger it is.
+    const int64_t input_bytes = n_subs * kSubBytes + n_elements;
+    return input_bytes < kMaxInputBytesForPlainLoads ? kDeepSmall : kDeep;
   }
   if (elems_per_sub < kMinElemsPerSubForDeepest) return kDeep;
   return kDeepest;
