@@ -39,7 +39,8 @@ extern "C" {
 #define DF11_SUBBLOCK_BYTES 512
 #define DF11_MAX_ELEMS_PER_SUBBLOCK 4096
 
-/* Version of this interface: 3 = df11_decode_static_workspace added, workspace holds fused LUT rows. */
+/* Version of this interface: 3 = df11_decode_static_workspace, df11_force_launch_plan and
+ * df11_launch_plan_name added, workspace holds fused LUT rows. */
 int df11_version(void);
 const char *df11_error_string(int code);
 
