@@ -224,10 +224,16 @@ def main():
         step()
     torch.cuda.synchronize()
     if a.calibration_copy:
+        import ctypes
+        from dfloat11_amd import build as B
+        copy_lib = ctypes.CDLL(B.CALIBRATION_LIB)   # built by build(); not part of the decode library
+        copy_lib.calibration_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         src = torch.zeros(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
         for _ in range(5):
-            D.calibration_copy(src, dst)
+            rc = copy_lib.calibration_copy(src.data_ptr(), dst.data_ptr(), src.numel(), stream_handle)
+            if rc != 0:
+                raise RuntimeError(f"calibration_copy failed: {rc}")
         torch.cuda.synchronize()
         del src, dst
     # The timed region: K steps launched back to back, between two HIP events on the

@@ -54,12 +54,10 @@ def hip_lib():
         L.df11_decode.restype = _i32
         L.df11_decode_static_workspace.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i32, _vp]
         L.df11_decode_static_workspace.restype = _i32
-        L.df11_force_launch_plan.argtypes = [_i32]
-        L.df11_force_launch_plan.restype = _i32
+        L.df11_decode_with_plan.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp, _i32]
+        L.df11_decode_with_plan.restype = _i32
         L.df11_launch_plan_name.argtypes = [_i64, _i64, _i32]
         L.df11_launch_plan_name.restype = ctypes.c_char_p
-        L.df11_calibration_copy.argtypes = [_vp, _vp, _i64, _vp]
-        L.df11_calibration_copy.restype = _i32
         _hip = L
     return _hip
 

@@ -1,7 +1,9 @@
 """Compiles the native libraries in-tree.
 
-libdf11_hip.so    HIP kernels + device C-ABI, hipcc --offload-arch=gfx950
-libdf11_codec.so  host codec C-ABI, g++
+libdf11_hip.so          HIP kernels + device C-ABI, hipcc --offload-arch=gfx950
+libdf11_codec.so        host codec C-ABI, g++
+libcalibration_copy.so  a plain copy kernel for the benchmark's counter calibration (no part
+                        of the interface; nothing in the package loads it)
 """
 import os
 import shutil
@@ -11,6 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 HIP_LIB = os.path.join(HERE, "libdf11_hip.so")
 CODEC_LIB = os.path.join(HERE, "libdf11_codec.so")
+CALIBRATION_LIB = os.path.join(HERE, "libcalibration_copy.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -35,6 +38,16 @@ def build_hip(verbose=False):
     return HIP_LIB
 
 
+def build_calibration(verbose=False):
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-o", CALIBRATION_LIB, os.path.join(CSRC, "calibration_copy.hip")]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
+    if verbose:
+        print(" ".join(cmd))
+    return CALIBRATION_LIB
+
+
 def build_codec(verbose=False):
     cmd = [shutil.which("g++") or "g++", *CXX_FLAGS, "-o", CODEC_LIB, os.path.join(CSRC, "df11_codec.cpp")]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -46,7 +59,7 @@ def build_codec(verbose=False):
 
 
 def build_all(verbose=False):
-    return build_hip(verbose), build_codec(verbose)
+    return build_hip(verbose), build_codec(verbose), build_calibration(verbose)
 
 
 if __name__ == "__main__":

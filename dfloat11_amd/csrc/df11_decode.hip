@@ -26,7 +26,6 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include <atomic>
 #include <mutex>
 
 #include "../../include/df11.h"
@@ -548,8 +547,6 @@ constexpr int kMinElemsPerSubForDeepest = 2560;
 constexpr int kMaxRoundsForPhasePriority = 16;
 constexpr int64_t kMaxInputBytesForPlainLoads = 40 << 20;   // about 30 M weight-like elements
 
-std::atomic<int> g_forced_plan{-1};   // df11_force_launch_plan: -1 = choose per stream
-
 const LaunchPlan kWide{decode_kernel_wide, kWideGroupsPerCu, nullptr, "wide", nullptr};
 const LaunchPlan kDeep{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short, "deep", "deep/short"};
 const LaunchPlan kDeepSmall{decode_kernel_deep_small, kDeepGroupsPerCu, decode_kernel_deep_small, "deep/small",
@@ -557,8 +554,9 @@ const LaunchPlan kDeepSmall{decode_kernel_deep_small, kDeepGroupsPerCu, decode_k
 const LaunchPlan kDeepest{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short, "deepest",
                           "deepest/short"};
 
-LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
-  switch (g_forced_plan.load(std::memory_order_relaxed)) {
+// `pinned` is one of DF11_PLAN_*: anything but a plan's number leaves the choice to the rule.
+LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned = DF11_PLAN_AUTO) {
+  switch (pinned) {
     case DF11_PLAN_WIDE: return kWide;
     case DF11_PLAN_DEEP: return kDeep;
     case DF11_PLAN_DEEPEST: return kDeepest;
@@ -591,15 +589,6 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus) {
 
 bool few_rounds(int64_t n_subs, int64_t grid) {
   return n_subs <= (int64_t)kMaxRoundsForPhasePriority * grid * kWavesPerGroup;
-}
-
-// Plain streaming copy, 16 bytes per lane: the known-traffic kernel against
-// which hardware byte counters are calibrated.
-__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src,
-                                                   uint4* __restrict__ dst, int64_t n_vec) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec;
-       i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = src[i];
 }
 
 struct DeviceInfo {
@@ -677,7 +666,7 @@ int enqueue_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const 
 int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
                    const uint8_t* gaps, uint16_t* outputs, int32_t n_luts, int64_t n_bytes,
                    int64_t n_elements, const uint8_t* ws, int32_t max_elems_per_subblock,
-                   const DeviceInfo& info, hipStream_t s) {
+                   const DeviceInfo& info, hipStream_t s, int pinned_plan = DF11_PLAN_AUTO) {
   if (max_elems_per_subblock <= 0 || max_elems_per_subblock > kMaxElemsPerSub)
     max_elems_per_subblock = kMaxElemsPerSub;
   DecodeSizes z;
@@ -695,7 +684,7 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
   const size_t lds_bytes = (size_t)kLdsSkip + (size_t)tables_bytes(n_rows) +
                            (size_t)kWavesPerGroup * (size_t)z.stage_cap;
-  const LaunchPlan plan = plan_launch(z.n_subs, n_elements, info.cus);
+  const LaunchPlan plan = plan_launch(z.n_subs, n_elements, info.cus, pinned_plan);
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, plan.groups_per_cu);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
@@ -742,7 +731,7 @@ int scratch_of_current_device(uint8_t** out) {
 
 extern "C" {
 
-int df11_version(void) { return 3; }
+int df11_version(void) { return 4; }
 
 const char* df11_error_string(int code) {
   switch (code) {
@@ -793,12 +782,6 @@ int df11_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const uin
   return DF11_OK;
 }
 
-int df11_force_launch_plan(int plan) {
-  if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_DEEPEST) return DF11_ERR_INVALID_ARGUMENT;
-  g_forced_plan.store(plan, std::memory_order_relaxed);
-  return DF11_OK;
-}
-
 const char* df11_launch_plan_name(int64_t n_bytes, int64_t n_elements, int32_t compute_units) {
   if (n_bytes <= 0 || n_elements <= 0 || compute_units <= 0) return "";
   const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
@@ -809,24 +792,10 @@ const char* df11_launch_plan_name(int64_t n_bytes, int64_t n_elements, int32_t c
   return few_rounds(n_subs, grid) && plan.kernel_short ? plan.name_short : plan.name;
 }
 
-int df11_calibration_copy(const void* src, void* dst, int64_t n_bytes, void* stream) {
-  if (!src || !dst || n_bytes <= 0 || (n_bytes & 15)) return DF11_ERR_INVALID_ARGUMENT;
-  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15)
-    return DF11_ERR_INVALID_ARGUMENT;
-  DeviceInfo info;
-  if (int rc = device_info(info)) return rc;
-  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)(info.cus * 8)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint4*>(src),
-                     static_cast<uint4*>(dst), n_bytes / 16);
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? DF11_OK : hip_fail(e);
-}
-
-int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
-                const uint32_t* output_positions, const uint8_t* gaps, uint16_t* outputs,
-                int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void* workspace,
-                int32_t max_elems_per_subblock, void* stream) {
-  (void)output_positions;   // superseded by the sub-block positions in the workspace
+namespace {
+int checked_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
+                   const uint8_t* gaps, uint16_t* outputs, int32_t n_luts, int64_t n_bytes, int64_t n_elements,
+                   const void* workspace, int32_t max_elems_per_subblock, void* stream, int pinned_plan) {
   if (n_bytes < 0 || n_elements < 0 || n_luts < 2) return DF11_ERR_INVALID_ARGUMENT;
   if (n_bytes == 0 || n_elements == 0) return DF11_OK;
   if (!luts || !encoded_exponent || !sign_mantissa || !gaps || !outputs || !workspace)
@@ -838,7 +807,27 @@ int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint
   if (int rc = device_info(info)) return rc;
   return enqueue_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements,
                         static_cast<const uint8_t*>(workspace), max_elems_per_subblock, info,
-                        static_cast<hipStream_t>(stream));
+                        static_cast<hipStream_t>(stream), pinned_plan);
+}
+}  // namespace
+
+int df11_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
+                const uint32_t* output_positions, const uint8_t* gaps, uint16_t* outputs,
+                int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void* workspace,
+                int32_t max_elems_per_subblock, void* stream) {
+  (void)output_positions;   // superseded by the sub-block positions in the workspace
+  return checked_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements, workspace,
+                        max_elems_per_subblock, stream, DF11_PLAN_AUTO);
+}
+
+int df11_decode_with_plan(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
+                          const uint32_t* output_positions, const uint8_t* gaps, uint16_t* outputs,
+                          int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void* workspace,
+                          int32_t max_elems_per_subblock, void* stream, int32_t plan) {
+  (void)output_positions;
+  if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_DEEPEST) return DF11_ERR_INVALID_ARGUMENT;
+  return checked_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements, workspace,
+                        max_elems_per_subblock, stream, plan);
 }
 
 int df11_decode_static_workspace(const uint8_t* luts, const uint8_t* encoded_exponent,

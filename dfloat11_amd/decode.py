@@ -100,9 +100,14 @@ def prepare(luts, encoded_exponent, output_positions, gaps, n_elements, workspac
     return workspace, int(max_sub.value)
 
 
+PLANS = {"auto": -1, "wide": 0, "deep": 1, "deepest": 2}
+
+
 def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,
-           max_elems_per_subblock=0):
-    """Decode one DF11 stream into `out` (bfloat16, >= n_elements) on the current stream."""
+           max_elems_per_subblock=0, plan=None):
+    """Decode one DF11 stream into `out` (bfloat16, >= n_elements) on the current stream.
+    `plan` (a key or value of PLANS) pins the kernel's launch plan for this call only (tests
+    and measurements); by default the library chooses per stream."""
     _require_cuda(luts=luts, encoded_exponent=encoded_exponent, sign_mantissa=sign_mantissa,
                   output_positions=output_positions, gaps=gaps, out=out, workspace=workspace)
     _check_stream_tensors(luts, encoded_exponent, output_positions, gaps)
@@ -112,13 +117,16 @@ def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, w
         raise _native.DF11Error("out must be a bfloat16 tensor with at least n_elements elements")
     if workspace.numel() * workspace.element_size() < workspace_bytes(n_bytes):
         raise _native.DF11Error("workspace buffer too small")
-    with torch.cuda.device(out.device):
-        rc = _native.hip_lib().df11_decode(
-            luts.data_ptr(), encoded_exponent.data_ptr(), sign_mantissa.data_ptr(),
+    args = (luts.data_ptr(), encoded_exponent.data_ptr(), sign_mantissa.data_ptr(),
             output_positions.data_ptr(), gaps.data_ptr(), out.data_ptr(),
-            luts.shape[0], n_bytes, n_elements, workspace.data_ptr(), int(max_elems_per_subblock),
-            _stream_ptr(out.device))
-    _native.check(rc, "df11_decode")
+            luts.shape[0], n_bytes, n_elements, workspace.data_ptr(), int(max_elems_per_subblock))
+    with torch.cuda.device(out.device):
+        if plan is None:
+            rc = _native.hip_lib().df11_decode(*args, _stream_ptr(out.device))
+        else:
+            rc = _native.hip_lib().df11_decode_with_plan(*args, _stream_ptr(out.device),
+                                                         int(PLANS.get(plan, plan)))
+    _native.check(rc, "df11_decode" if plan is None else "df11_decode_with_plan")
     return out
 
 
@@ -151,15 +159,3 @@ def launch(bound, device):
             rc = lib.df11_decode(*bound, torch.cuda.current_stream(device).cuda_stream)
     if rc:
         _native.check(rc, "df11_decode")
-
-
-def calibration_copy(src, dst):
-    """Streaming copy of known size (profiler byte-counter calibration)."""
-    _require_cuda(src=src, dst=dst)
-    n = src.numel() * src.element_size()
-    if dst.numel() * dst.element_size() != n:
-        raise _native.DF11Error("src and dst differ in size")
-    with torch.cuda.device(src.device):
-        rc = _native.hip_lib().df11_calibration_copy(src.data_ptr(), dst.data_ptr(), n, _stream_ptr(src.device))
-    _native.check(rc, "df11_calibration_copy")
-    return dst

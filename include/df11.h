@@ -39,8 +39,9 @@ extern "C" {
 #define DF11_SUBBLOCK_BYTES 512
 #define DF11_MAX_ELEMS_PER_SUBBLOCK 4096
 
-/* Version of this interface: 3 = df11_decode_static_workspace, df11_force_launch_plan and
- * df11_launch_plan_name added, workspace holds fused LUT rows. */
+/* Version of this interface: 4 = df11_decode_with_plan replaces the process-wide
+ * df11_force_launch_plan, df11_calibration_copy removed (3 = df11_decode_static_workspace
+ * and df11_launch_plan_name added, workspace holds fused LUT rows). */
 int df11_version(void);
 const char *df11_error_string(int code);
 
@@ -122,20 +123,27 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
                                  int32_t max_elems_per_subblock, void *stream);
 
 /*
- * The decode kernel exists in three launch plans (workgroups resident per CU and
- * depth of its requests for sign_mantissa bytes); df11_decode picks one per
- * stream from its size and its elements per 512 bytes of bitstream (and, within
- * the two plans for large streams, how wavefront priorities are set from the
- * stream's size, which this call leaves alone).  This call
- * pins the plan for every later decode of the process, or hands the choice back
- * (DF11_PLAN_AUTO).  Testing and measurement aid with no counterpart in the
- * reference: every plan decodes every stream to the same bits.
+ * df11_decode with the launch plan chosen by the caller.  The decode kernel is
+ * compiled for three launch plans (workgroups resident per CU and how far ahead
+ * it requests sign_mantissa bytes: DF11_PLAN_WIDE, _DEEP, _DEEPEST; the two plans
+ * for large streams come in further compilations that differ in how wavefront
+ * priorities are set and in the cache policy of the loads, which the stream's
+ * size decides in either entry point).  df11_decode picks the plan per stream from
+ * its size and its elements per 512 bytes of bitstream; this entry point takes it
+ * as an argument, for tests that drive every stream through every plan and for
+ * measurements.  DF11_PLAN_AUTO behaves as df11_decode does.  The choice is local
+ * to the call: nothing in the library remembers it.  No counterpart in the
+ * reference; every plan decodes every stream to the same bits.
  */
 #define DF11_PLAN_AUTO (-1)
 #define DF11_PLAN_WIDE 0
 #define DF11_PLAN_DEEP 1
 #define DF11_PLAN_DEEPEST 2
-int df11_force_launch_plan(int plan);
+int df11_decode_with_plan(const uint8_t *luts, const uint8_t *encoded_exponent,
+                          const uint8_t *sign_mantissa, const uint32_t *output_positions,
+                          const uint8_t *gaps, uint16_t *outputs, int32_t n_luts, int64_t n_bytes,
+                          int64_t n_elements, const void *workspace,
+                          int32_t max_elems_per_subblock, void *stream, int32_t plan);
 
 /*
  * Which compilation of the decode kernel df11_decode launches for a stream of
@@ -146,13 +154,6 @@ int df11_force_launch_plan(int plan);
  * counterpart in the reference.
  */
 const char *df11_launch_plan_name(int64_t n_bytes, int64_t n_elements, int32_t compute_units);
-
-/*
- * Streaming device copy of n_bytes (multiple of 16, both pointers 16-byte
- * aligned).  Measurement aid with no counterpart in the reference: a kernel of
- * known HBM traffic against which profiler byte counters are calibrated.
- */
-int df11_calibration_copy(const void *src, void *dst, int64_t n_bytes, void *stream);
 
 /* -------------------------------------------------------------- Host codec */
 

@@ -25,7 +25,7 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_error_strings():
     hip = _native.hip_lib()
-    assert hip.df11_version() == 3
+    assert hip.df11_version() == 4
     assert hip.df11_error_string(0) == b"ok"
     assert hip.df11_error_string(-1) == b"invalid argument"
     # header + tables + 17 fused LUT rows + (8 sub-blocks per 4096-byte block + 1) positions, rounded to 16
@@ -73,11 +73,16 @@ def test_plain_c_caller_builds_against_the_header():
     assert "libdf11_hip.so" in out and "libdf11_codec.so" in out and "not found" not in out
 
 
-def test_launch_plan_override_is_validated():
+def test_plan_argument_is_validated_before_anything_else():
+    """df11_decode_with_plan rejects a plan number it does not know; the check comes first, so
+    no GPU and no valid pointers are needed to see it.  No call changes what a later call does:
+    the library keeps no launch state."""
     hip = _native.hip_lib()
-    assert hip.df11_force_launch_plan(3) == -1 and hip.df11_force_launch_plan(-2) == -1
-    for plan in (0, 1, 2, -1):
-        assert hip.df11_force_launch_plan(plan) == 0
+    for plan in (3, -2, 100):
+        assert hip.df11_decode_with_plan(None, None, None, None, None, None, 2, 16, 16, None, 0, None, plan) == -1
+    # an empty stream is a successful no-op under every plan
+    for plan in (-1, 0, 1, 2):
+        assert hip.df11_decode_with_plan(None, None, None, None, None, None, 2, 0, 0, None, 0, None, plan) == 0
 
 
 def test_launch_plan_follows_stream_size_and_code_lengths():
@@ -106,9 +111,3 @@ def test_launch_plan_follows_stream_size_and_code_lengths():
         assert plan(n, 1.16) == "wide"                 # decode-bound whatever the size
     assert plan(4096 * 14336, cus=64) == "deep"        # the same matrix is 36 rounds on a quarter of the CUs
     assert hip.df11_launch_plan_name(0, 10, 256) == b"" and hip.df11_launch_plan_name(10, 10, 0) == b""
-    # a pinned plan answers for itself
-    assert hip.df11_force_launch_plan(0) == 0
-    try:
-        assert plan(218_103_808) == "wide"
-    finally:
-        assert hip.df11_force_launch_plan(-1) == 0

@@ -30,7 +30,7 @@ def to_gpu(c, pad_front=0):
     return g
 
 
-def gpu_decode(c, max_elems=None, pad_front=0, out=None):
+def gpu_decode(c, max_elems=None, pad_front=0, out=None, plan=None):
     g = to_gpu(c, pad_front)
     n = c["sign_mantissa"].size
     ws, max_sub = D.prepare(g["luts"].contiguous(), g["encoded_exponent"], g["output_positions"],
@@ -40,7 +40,7 @@ def gpu_decode(c, max_elems=None, pad_front=0, out=None):
     if max_elems is None:
         max_elems = max_sub
     D.decode(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
-             out, ws, max_elems)
+             out, ws, max_elems, plan=plan)
     torch.cuda.synchronize()
     return out.view(torch.int16).cpu().numpy().view(np.uint16)[:n]
 
@@ -58,25 +58,12 @@ def test_gpu_matches_oracle(oracle, kind, n):
     assert np.array_equal(got, w)
 
 
-@pytest.fixture()
-def launch_plan():
-    """Pins one of the decode kernel's launch plans for a test and hands the choice back after it."""
-    from dfloat11_amd import _native
-    lib = _native.hip_lib()
-
-    def force(plan):
-        assert lib.df11_force_launch_plan(plan) == 0
-    yield force
-    assert lib.df11_force_launch_plan(-1) == 0
-
-
 @pytest.mark.parametrize("plan", [0, 1, 2], ids=["wide", "deep", "deepest"])
-def test_gpu_every_launch_plan_matches_oracle(oracle, launch_plan, plan):
+def test_gpu_every_launch_plan_matches_oracle(oracle, plan):
     """The plans differ in resident workgroups and in how many groups of sign|mantissa
     bytes are requested early; the automatic choice sends small streams to one of them
-    only.  Pinned, each plan decodes every kind, ragged sizes, unaligned buffers and the
-    worst-case staging to the oracle's bits."""
-    launch_plan(plan)
+    only.  Through df11_decode_with_plan each plan decodes every kind, ragged sizes,
+    unaligned buffers and the worst-case staging to the oracle's bits."""
     for kind in KINDS:
         for n in (1, 511, 4097, 70_001, 300_000):
             print(f"case plan={plan} kind={kind} n={n}", flush=True)
@@ -84,21 +71,21 @@ def test_gpu_every_launch_plan_matches_oracle(oracle, launch_plan, plan):
             c = compress_product(w)
             ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"],
                                   c["output_positions"], c["gaps"])
-            assert np.array_equal(gpu_decode(c), ref), (kind, n)
+            assert np.array_equal(gpu_decode(c, plan=plan), ref), (kind, n)
             assert np.array_equal(ref, w)
     w = make_case("laplace", 120_000, 79)
     c = compress_product(w)
     for pad in (1, 4, 7):
-        assert np.array_equal(gpu_decode(c, pad_front=pad), w), pad
+        assert np.array_equal(gpu_decode(c, pad_front=pad, plan=plan), w), pad
     buf = torch.zeros(w.size + 16, dtype=torch.bfloat16, device=DEV)
     for shift in (1, 3, 8):
         buf.zero_()
-        assert np.array_equal(gpu_decode(c, out=buf[shift:shift + w.size]), w)
+        assert np.array_equal(gpu_decode(c, out=buf[shift:shift + w.size], plan=plan), w)
         whole = buf.view(torch.int16).cpu().numpy()
         assert not whole[:shift].any() and not whole[shift + w.size:].any()
     for kind in ("normal", "zeros", "fib"):
         w = make_case(kind, 200_000, 67)
-        assert np.array_equal(gpu_decode(compress_product(w), max_elems=0), w), kind
+        assert np.array_equal(gpu_decode(compress_product(w), max_elems=0, plan=plan), w), kind
 
 
 def test_gpu_random_codes_and_fillings(oracle):
