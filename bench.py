@@ -83,7 +83,8 @@ def cpu_baseline(stream, original_u16, budget_s=12.0):
     first, last = int(pos[0]), int(pos[min(sample, pos.size - 1)])
     bit_exact = bool(np.array_equal(out[first:last], original_u16[first:last]))
     return {
-        "value": bytes_done / dt / 1e9, "unit": "GB/s", "cores": n_threads, "kind": "port",
+        "value": bytes_done / dt / 1e9, "unit": "GB/s", "cores": n_threads, "host_cores": os.cpu_count(),
+        "host_cores_usable": len(os.sched_getaffinity(0)), "kind": "port",
         "bit_exact": bit_exact,
         "sample": f"first {sample} of {n_blocks} bitstream blocks of the same stream ({elems} elements), "
                   f"median of {repeats} passes of {dt:.2f} s, scalar C restatement of the reference "
@@ -92,27 +93,92 @@ def cpu_baseline(stream, original_u16, budget_s=12.0):
     }
 
 
-def side_measurements(torch, dev, steps=30, warmup=30):
+def side_measurements(torch, dev, embedding_shape=True):
     """Kernel-time throughput of the same entry point on other inputs: the 4096x14336
-    matrix under each adversarial exponent distribution, and N(0, 0.02) tensors of the
-    sizes a per-Linear compression produces.  Returns (mixes, sizes): name -> figures."""
+    matrix (and the 151936x4096 embedding-shaped tensor) under each adversarial exponent
+    distribution, and N(0, 0.02) tensors of the sizes a per-Linear compression produces.
+    Every stream is held in enough device copies, decoded in turn, that no launch finds its
+    input in the 256 MB memory-side cache: `hbm_frac` is HBM-fed; the figures for one copy
+    decoded over and over are reported beside it as `same_copy_*`.
+    Returns (mixes, sizes): name -> figures."""
     import bench_extra
-    keep = ("n_elements", "kernel_ms_median", "GBps", "hbm_frac", "back_to_back_ms_per_launch",
-            "back_to_back_hbm_frac", "bit_exact", "bits_per_exponent", "max_code_bits", "compressed_over_bf16")
+
+    def figures(w):
+        r = bench_extra.time_copies_in_turn(torch, w)
+        return {"n_elements": r["n_elements"], "kernel": r["kernel"], "device_copies": r["device_copies"],
+                "ms_per_launch": r["copies_in_turn_ms_per_launch"],
+                "GBps": r["algorithmic_bytes"] / (r["copies_in_turn_ms_per_launch"] * 1e-3) / 1e9,
+                "hbm_frac": r["copies_in_turn_hbm_frac"],
+                "same_copy_ms_per_launch": r["same_copy_ms_per_launch"], "same_copy_frac": r["same_copy_hbm_frac"],
+                "bit_exact": r["bit_exact"], "bits_per_exponent": r["bits_per_exponent"],
+                "max_code_bits": r["max_code_bits"], "compressed_over_bf16": r["compressed_over_bf16"]}
+
     mixes, sizes = {}, {}
-    for kind in ("laplace", "outliers", "uniform256", "zeros"):
-        w = bench_extra.make_mix(torch, kind, 4096 * 14336, dev, seed=7)
-        r = bench_extra.time_decode(torch, w, steps, warmup)
-        mixes[f"{kind} 4096x14336"] = {k: r[k] for k in keep}
-        del w
+    shapes = [(4096, 14336)] + ([(151936, 4096)] if embedding_shape else [])
+    for rows, cols in shapes:
+        for kind in ("laplace", "outliers", "uniform256", "zeros"):
+            w = bench_extra.make_mix(torch, kind, rows * cols, dev, seed=7)
+            mixes[f"{kind} {rows}x{cols}"] = figures(w)
+            del w
+            torch.cuda.empty_cache()
     for rows, cols in ((4096, 4096), (4096, 14336)):
         g = torch.Generator(device=dev).manual_seed(0)
         w = (torch.randn(rows * cols, generator=g, device=dev) * 0.02).to(torch.bfloat16)
-        r = bench_extra.time_decode(torch, w, steps, warmup)
-        sizes[f"normal {rows}x{cols}"] = {k: r[k] for k in keep}
+        sizes[f"normal {rows}x{cols}"] = figures(w)
         del w
     torch.cuda.empty_cache()
     return mixes, sizes
+
+
+def end_to_end(torch, dev, num_tokens, batch_sizes=(1, 64)):
+    """Generation with the Qwen3-8B-shaped model (random-init, greedy, 64 random prompt ids)
+    in BF16 and with every linear and the embedding in DF11, at each batch size: tokens per
+    second of both, their ratio, peak device memory, and whether logits and tokens are
+    identical.  Same fields as the reference's benchmark script prints
+    (reference: inference.py:62-97)."""
+    from dfloat11_amd import inference
+    t0 = time.perf_counter()
+    out = {}
+    for r in inference.compare_synthetic("qwen3-8b", list(batch_sizes), num_tokens, prompt_len=64, device=dev):
+        out[f"batch {r['batch_size']}"] = {
+            "new_tokens": r["num_tokens"], "prompt_len": r["prompt_len"],
+            "bf16_tokens_per_second": r["bf16"]["tokens_per_second"],
+            "df11_tokens_per_second": r["df11"]["tokens_per_second"],
+            "df11_over_bf16": r["df11_over_bf16_tokens_per_second"],
+            "bf16_peak_memory_mb": r["bf16"]["gpu_peak_memory_mb"],
+            "df11_peak_memory_mb": r["df11"]["gpu_peak_memory_mb"],
+            "logits_bit_identical": r["logits_bit_identical"], "tokens_identical": r["tokens_identical"]}
+        out["model"] = r["model"]
+        out["compressed_over_bf16"] = r["compressed_over_bf16"]
+        out["compress_seconds_host"] = r["compress_seconds"]
+    out["leg_seconds"] = time.perf_counter() - t0
+    return out
+
+
+def offload(torch, dev, double_blocks, single_blocks):
+    """One pass over a FLUX.1-dev-shaped block stack (hidden 3072, 4096 image + 512 text
+    tokens) in BF16, with resident DF11 streams, and with the streams in pinned host memory
+    copied one block ahead of use (cpu_offload): time per pass, peak device memory, what a
+    block costs when nothing overlaps (host-to-device copy, then decode), how well the copies
+    overlap, and whether the outputs are identical."""
+    import types
+
+    import bench_extra
+    t0 = time.perf_counter()
+    a = types.SimpleNamespace(double_blocks=double_blocks, single_blocks=single_blocks, image_tokens=4096,
+                              text_tokens=512)
+    r = bench_extra.flux_report(a, torch, dev, passes=6)
+    out = {"double_blocks": double_blocks, "single_blocks": single_blocks, "hidden": 3072,
+           "image_tokens": 4096, "text_tokens": 512, "parameters": r["config"]["parameters"]}
+    for key, run in r["passes"].items():
+        out[key] = {"ms_per_pass": run["steady_pass_s"] * 1e3, "peak_device_memory_mb": run["peak_device_memory_mb"]}
+    out["per_block_unoverlapped"] = [
+        {"block": b["block"], "n_elements": b["n_elements"], "host_to_device_ms": b["h2d_ms"],
+         "host_to_device_GBps": b["h2d_GBps"], "decode_ms": b["decode_ms"]} for b in r["per_block_serial"]]
+    out["overlap_efficiency"] = r["overlap_efficiency"]
+    out["outputs_bit_identical"] = r["outputs_bit_identical"]
+    out["leg_seconds"] = time.perf_counter() - t0
+    return out
 
 
 def profiled_traffic():
@@ -141,6 +207,15 @@ def main():
                          "run at the clock the device settles at under load, whatever --warmup is")
     ap.add_argument("--no-mixes", action="store_true",
                     help="skip the per-distribution and per-size side measurements (config.mixes, config.sizes)")
+    ap.add_argument("--no-embedding-mixes", action="store_true",
+                    help="config.mixes on the 4096x14336 matrix only, not on the 151936x4096 tensor as well")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip config.e2e: Qwen3-8B-shaped generation, BF16 against DF11, batch 1 and 64 (about 1 min)")
+    ap.add_argument("--e2e-tokens", type=int, default=64, help="new tokens per sequence in config.e2e")
+    ap.add_argument("--no-offload", action="store_true",
+                    help="skip config.offload: FLUX-shaped block stack with cpu_offload (about 20 s)")
+    ap.add_argument("--offload-blocks", type=int, nargs=2, default=(4, 8), metavar=("DOUBLE", "SINGLE"),
+                    help="double-stream and single-stream blocks of the config.offload stack (the full model: 19 38)")
     ap.add_argument("--copies", type=int, default=4,
                     help="device copies of the compressed block that the steps decode in turn")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -322,7 +397,8 @@ def main():
         copies.clear()
         out = None
         torch.cuda.empty_cache()
-        result["config"]["mixes"], result["config"]["sizes"] = side_measurements(torch, dev)
+        result["config"]["mixes"], result["config"]["sizes"] = side_measurements(
+            torch, dev, embedding_shape=not a.no_embedding_mixes)
         if not all(m["bit_exact"] for m in list(result["config"]["mixes"].values())
                    + list(result["config"]["sizes"].values())):
             result["error"] = "a side measurement did not decode bit-exactly"
@@ -333,6 +409,19 @@ def main():
         result["cpu_baseline"] = cpu_baseline(stream, w_cpu.view(torch.int16).numpy().view(np.uint16))
         if not result["cpu_baseline"]["bit_exact"]:
             result["error"] = "the CPU oracle's output differs from the original block"
+            bit_exact = False
+    copies.clear()
+    out = None
+    torch.cuda.empty_cache()
+    if not a.no_e2e:
+        result["config"]["e2e"] = e2e = end_to_end(torch, dev, a.e2e_tokens)
+        if not all(v["logits_bit_identical"] and v["tokens_identical"] for k, v in e2e.items() if k.startswith("batch")):
+            result["error"] = "DF11 generation differs from BF16"
+            bit_exact = False
+    if not a.no_offload:
+        result["config"]["offload"] = off = offload(torch, dev, *a.offload_blocks)
+        if not all(off["outputs_bit_identical"].values()):
+            result["error"] = "offloaded pass differs from the resident one"
             bit_exact = False
     if bit_exact is False and "error" not in result:
         result["error"] = "decoded block differs from the original"

@@ -184,8 +184,11 @@ def time_copies_in_turn(torch, w, launches=40, preheat_ms=150.0):
     same = per_launch(lambda i: 0)
     algo = algorithmic_bytes(enc.numel(), n, luts.shape[0])
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    lengths = luts[-1].numpy()
     return {
         "n_elements": n, "bitstream_sub_blocks": -(-enc.numel() // 512), "algorithmic_bytes": algo,
+        "bits_per_exponent": 8.0 * enc.numel() / n, "max_code_bits": int(lengths.max()),
+        "compressed_over_bf16": input_bytes / (2.0 * n),
         "kernel": "decode_kernel_" + lib.df11_launch_plan_name(int(enc.numel()), int(n), cus).decode().replace("/", "_"),
         "device_copies": n_copies, "copies_in_turn_ms_per_launch": in_turn,
         "copies_in_turn_hbm_frac": algo / (in_turn * 1e-3) / 1e9 / HBM_PEAK_GBPS,

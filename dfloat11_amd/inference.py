@@ -131,6 +131,73 @@ def timed_generate(model, inputs, num_tokens, do_sample):
     }
 
 
+def _random_prompts(model, batch_size, prompt_len, seed, device):
+    import torch
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    ids = torch.randint(0, model.config.vocab_size, (batch_size, prompt_len), generator=gen).to(device)
+    return {"input_ids": ids, "attention_mask": torch.ones_like(ids)}
+
+
+def compare_synthetic(shape, batch_sizes, num_tokens, prompt_len=64, seed=42, device="cuda:0", layers=None):
+    """Builds the named architecture once with random-init BF16 weights, generates
+    greedily at every batch size, compresses the model in memory and generates again
+    from the same prompts.  Returns one report per batch size with the fields of the
+    reference's benchmark for both models (reference: inference.py:62-97), their
+    ratio, and whether logits and tokens are identical."""
+    import torch
+    device = torch.device(device)
+    model = build_synthetic(shape, device, seed, layers)
+    name = f"{shape} (random-init N(0, 0.02), {sum(p.numel() for p in model.parameters())/1e9:.2f} B parameters)"
+    reports, kept = [], []
+    for b in batch_sizes:
+        inputs = _random_prompts(model, b, prompt_len, seed, device)
+        with torch.no_grad():
+            ref_logits = model(**inputs, use_cache=False).logits
+        timed_generate(model, inputs, min(8, num_tokens), False)           # warm-up
+        ref_out, stats = timed_generate(model, inputs, num_tokens, False)
+        reports.append({"batch_size": b, "num_tokens": num_tokens, "model": name, "prompt_len": prompt_len,
+                        "bf16": stats})
+        kept.append((inputs, ref_logits.cpu(), ref_out))
+        del ref_logits
+    t0 = time.time()
+    compressed, original = convert_in_memory(model, LLM_PATTERNS, device)
+    compress_seconds = time.time() - t0
+    torch.cuda.empty_cache()
+    for report, (inputs, ref_logits, ref_out) in zip(reports, kept):
+        report["compress_seconds"] = compress_seconds
+        report["compressed_over_bf16"] = compressed / original
+        # warm-up pass: first-use work (decode workspaces, library handles) stays out of the timing
+        with torch.no_grad():
+            logits = model(**inputs, use_cache=False).logits
+        timed_generate(model, inputs, min(8, num_tokens), False)
+        out, stats = timed_generate(model, inputs, num_tokens, False)
+        report["df11"] = stats
+        report["logits_bit_identical"] = bool(torch.equal(logits.cpu(), ref_logits))
+        report["tokens_identical"] = bool(torch.equal(out, ref_out))
+        report["df11_over_bf16_tokens_per_second"] = stats["tokens_per_second"] / report["bf16"]["tokens_per_second"]
+        del logits
+    del model
+    from . import dfloat11 as D
+    D.TensorManager.clear()
+    torch.cuda.empty_cache()
+    return reports
+
+
+def _print_report(report, as_json):
+    if as_json:
+        print(json.dumps(report))
+        return
+    for key, value in report.items():
+        if isinstance(value, dict):
+            print(f"[{key}]")
+            print(f"  Decoding Latency for {value['new_tokens_per_sequence']} tokens: {value['latency_s']:.4f} seconds")
+            print(f"  Tokens per second: {value['tokens_per_second']:.2f}")
+            print(f"  GPU Memory Allocated: {value['gpu_memory_allocated_mb']:.2f} MB")
+            print(f"  GPU Peak Memory Usage: {value['gpu_peak_memory_mb']:.2f} MB")
+        else:
+            print(f"{key}: {value}")
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--model_name_or_path", type=str, default=None)
@@ -158,19 +225,17 @@ def main(argv=None):
     torch.cuda.set_device(device)
     report = {"batch_size": a.batch_size, "num_tokens": a.num_tokens}
 
+    if a.synthetic and a.compare_bf16:
+        report = compare_synthetic(a.synthetic, [a.batch_size], a.num_tokens, a.prompt_len, a.seed, device,
+                                   a.layers)[0]
+        _print_report(report, a.json)
+        return report
     if a.synthetic:
         model = build_synthetic(a.synthetic, device, a.seed, a.layers)
-        gen = torch.Generator(device="cpu").manual_seed(a.seed)
-        ids = torch.randint(0, model.config.vocab_size, (a.batch_size, a.prompt_len), generator=gen).to(device)
-        inputs = {"input_ids": ids, "attention_mask": torch.ones_like(ids)}
+        inputs = _random_prompts(model, a.batch_size, a.prompt_len, a.seed, device)
         do_sample = False
         report["model"] = f"{a.synthetic} (random-init N(0, 0.02), {sum(p.numel() for p in model.parameters())/1e9:.2f} B parameters)"
         report["prompt_len"] = a.prompt_len
-        if a.compare_bf16:
-            with torch.no_grad():
-                ref_logits = model(**inputs, use_cache=False).logits
-            timed_generate(model, inputs, min(8, a.num_tokens), do_sample)           # warm-up
-            ref_out, report["bf16"] = timed_generate(model, inputs, a.num_tokens, do_sample)
         t0 = time.time()
         compressed, original = convert_in_memory(model, LLM_PATTERNS, device)
         report["compress_seconds"] = time.time() - t0
@@ -201,23 +266,7 @@ def main(argv=None):
     out, stats = timed_generate(model, inputs, a.num_tokens, do_sample)
     report["bf16_model" if (a.bf16 and not a.synthetic) else "df11"] = stats
 
-    if a.synthetic and a.compare_bf16:
-        report["logits_bit_identical"] = bool(torch.equal(logits, ref_logits))
-        report["tokens_identical"] = bool(torch.equal(out, ref_out))
-        report["df11_over_bf16_tokens_per_second"] = stats["tokens_per_second"] / report["bf16"]["tokens_per_second"]
-
-    if a.json:
-        print(json.dumps(report))
-    else:
-        for key, value in report.items():
-            if isinstance(value, dict):
-                print(f"[{key}]")
-                print(f"  Decoding Latency for {value['new_tokens_per_sequence']} tokens: {value['latency_s']:.4f} seconds")
-                print(f"  Tokens per second: {value['tokens_per_second']:.2f}")
-                print(f"  GPU Memory Allocated: {value['gpu_memory_allocated_mb']:.2f} MB")
-                print(f"  GPU Peak Memory Usage: {value['gpu_peak_memory_mb']:.2f} MB")
-            else:
-                print(f"{key}: {value}")
+    _print_report(report, a.json)
     return report
 
 
