@@ -400,41 +400,33 @@ DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo
 
 // ---- one decode per chunk, kept in registers -------------------------------------
 // The fast path decodes a chunk once.  The lookups of a chunk are few (each
-// resolves up to four codes), so their results fit in registers: kMain lookups
-// that stay inside the chunk plus kTailSlots for the codes that reach into the
-// look-ahead (a tail lookup may hold symbols of the next chunk as well: they are
-// the true next symbols of the stream).  Once the lane's output offset is known,
-// the symbols are replayed into the staging area with no further table access.
-// A chunk that needs more lookups than there are slots reports `overflow` and is
-// handled by count_chunk / emit_chunk instead.
-// A lookup inside the chunk consumes at least four bits unless a code that does
-// not fit the rest of the window follows (four one-bit codes), and lookups inside
-// the chunk start at bit 53 or before: 14 of them hold any chunk of codes that
-// short, and seven are enough for weight-like streams (2.6 bits per code, 3.3
-// codes per lookup); the kernel is compiled for both.
+// resolves up to four codes), so their results fit in registers: kMainSlots
+// lookups that stay inside the chunk plus kTailSlots for the codes that reach
+// into the look-ahead (a tail lookup may hold symbols of the next chunk as well:
+// they are the true next symbols of the stream).  Once the lane's output offset
+// is known, the symbols are replayed into the staging area with no further
+// table access.  A chunk that
+// needs more lookups than there are slots reports `overflow` and is handled by
+// count_chunk / emit_chunk instead.
 constexpr int kMainSlots = 7;
-constexpr int kMainSlotsShortCodes = 14;
 constexpr int kTailSlots = 2;
+constexpr int kSlots = kMainSlots + kTailSlots;
 
-template <int kMain>
 struct ChunkSyms {
-  static constexpr int kSlots = kMain + kTailSlots;
-  uint32_t syms[kSlots];       // symbol bytes of lookup i, first code in byte 0, unused bytes zero
+  uint32_t syms[kSlots];   // symbol bytes of lookup i, first code in byte 0, unused bytes zero
   uint32_t ends[kSlots - 1];   // symbols of the chunk up to and including lookup i
-  uint32_t count;              // codes that start in the chunk
-  bool overflow;               // ran out of slots: count and syms are incomplete
+  uint32_t count;          // codes that start in the chunk
+  bool overflow;           // ran out of slots: count and syms are incomplete
 };
 
-template <int kMain>
-DF11_HD ChunkSyms<kMain> decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
-                                           uint32_t next, uint32_t gap) {
-  constexpr int kSlots = ChunkSyms<kMain>::kSlots;
-  ChunkSyms<kMain> r;
+DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
+                                    uint32_t next, uint32_t gap) {
+  ChunkSyms r;
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   const uint64_t next31 = look_ahead(next);
   uint32_t c = gap, n = 0;
 #pragma unroll
-  for (int i = 0; i < kMain; ++i) {
+  for (int i = 0; i < kMainSlots; ++i) {
     r.syms[i] = 0;
     if (c <= 64u - (uint32_t)kK) {          // the lookup stays inside the chunk
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
@@ -460,7 +452,7 @@ DF11_HD ChunkSyms<kMain> decode_chunk_regs(const Tables& t, const Rows& l, uint3
   }
 #pragma unroll
   for (int i = 0; i < kTailSlots; ++i) {
-    r.syms[kMain + i] = 0;
+    r.syms[kMainSlots + i] = 0;
     if (todo) {
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
@@ -469,14 +461,14 @@ DF11_HD ChunkSyms<kMain> decode_chunk_regs(const Tables& t, const Rows& l, uint3
         syms = entry_symbol(long_code);
         meta = entry_meta(long_code);
       }
-      r.syms[kMain + i] = syms;
+      r.syms[kMainSlots + i] = syms;
       const uint32_t k = meta >> 8;
       const uint32_t take = k < todo ? k : todo;
       n += take;
       todo -= take;
       w <<= (meta & 63u);
     }
-    if (kMain + i < kSlots - 1) r.ends[kMain + i] = n;
+    if (kMainSlots + i < kSlots - 1) r.ends[kMainSlots + i] = n;
   }
   r.overflow = r.overflow || todo != 0u;
   r.count = n;
@@ -515,11 +507,10 @@ DF11_HD uint32_t align_bytes(uint32_t hi, uint32_t lo, uint32_t bytes) {
 // (-pos) & 3 bytes to the right of {symbols, 0}, which one instruction per word
 // does from -pos itself; a lookup that starts on a word boundary ORs zero into the
 // word before it.
-template <int kMain>
-DF11_HD void replay_chunk(const ChunkSyms<kMain>& r, LdsBytes stage, uint32_t at) {
+DF11_HD void replay_chunk(const ChunkSyms& r, LdsBytes stage, uint32_t at) {
   const uint32_t minus_at = 0u - at;
 #pragma unroll
-  for (int i = 0; i < ChunkSyms<kMain>::kSlots; ++i) {
+  for (int i = 0; i < kSlots; ++i) {
     // lookup i starts where the lookups before it end
     const uint32_t minus_pos = i == 0 ? minus_at : minus_at - r.ends[i - 1];
     LdsBytes w = stage + (~minus_pos & ~3u);               // (pos - 1) & ~3

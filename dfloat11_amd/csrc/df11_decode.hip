@@ -289,7 +289,7 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, int kMain>
+template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority>
 __device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
@@ -403,7 +403,7 @@ __device__ __forceinline__ void decode_body(
     // One decode per chunk, results held in registers.  If any lane of the
     // wavefront ran out of register slots, or may not write all its symbols (end
     // of the tensor), the wavefront takes the two-pass route instead.
-    const ChunkSyms<kMain> cs = decode_chunk_regs<kMain>(t, l, c.hi, c.lo, c.next, gap);
+    const ChunkSyms cs = decode_chunk_regs(t, l, c.hi, c.lo, c.next, gap);
     const bool all_fit = wave_all(!cs.overflow);
     const uint32_t count = all_fit ? cs.count : count_chunk(t, l, c.hi, c.lo, c.next, gap);
     const uint32_t incl = wave_inclusive_scan(count);
@@ -511,21 +511,20 @@ __device__ __forceinline__ void decode_body(
 // under 38 M elements that fit its rounds better than those of `wide` (a stream that
 // small may still sit in the memory-side cache).
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
-#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd, main_slots) \
+#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd)             \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
                                                                              waves_per_simd)))    \
   void name(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,         \
             const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,                         \
             const uint8_t* __restrict__ ws, const DecodeSizes z) {                                \
-    decode_body<prefetch, streaming, phase_priority, main_slots>(codes, sign_mantissa, gaps, out, \
-                                                                 ws, z);                          \
+    decode_body<prefetch, streaming, phase_priority>(codes, sign_mantissa, gaps, out, ws, z);     \
   }
-DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6, kMainSlots)
-DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4, kMainSlots)
-DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4, kMainSlots)
-DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4, kMainSlots)
-DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4, kMainSlotsShortCodes)
-DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4, kMainSlotsShortCodes)
+DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6)
+DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4)
+DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4)
+DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4)
 #undef DF11_DECODE_KERNEL
 
 typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);

@@ -87,14 +87,14 @@ extern "C" int df11_emul_prepare(const uint8_t* luts, const uint8_t* codes, cons
   return (int)max_sub;
 }
 
-// The decode kernel's steps for one compilation of it (kMain: lookups inside a chunk
-// that are kept in registers).
-template <int kMain>
-static int emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
-                       const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
-                       int n_luts, int64_t n_bytes, int64_t n_elements,
-                       int max_elems_per_sub, int grid, int codes_misalign,
-                       int out_misalign, int flags) {
+// Same data arguments as df11_decode (include/df11.h), host pointers; `grid`
+// plays gridDim.x (workgroups of eight wavefronts).  max_elems_per_sub <= 0
+// selects the worst case, as in the library.
+extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
+                                const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
+                                int n_luts, int64_t n_bytes, int64_t n_elements,
+                                int max_elems_per_sub, int grid, int codes_misalign,
+                                int out_misalign, int flags) {
   if (max_elems_per_sub <= 0 || max_elems_per_sub > kMaxElemsPerSub) max_elems_per_sub = kMaxElemsPerSub;
   const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
   const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
@@ -137,7 +137,7 @@ static int emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t*
 
   std::vector<Chunk> chunk(kLanes);
   std::vector<uint32_t> gap(kLanes), count(kLanes), excl(kLanes);
-  std::vector<ChunkSyms<kMain>> regs(kLanes);
+  std::vector<ChunkSyms> regs(kLanes);
   const bool force_two_pass = (flags & 1) != 0;   // exercise the fall-back route on any input
   const bool force_check = true;
   for (int64_t wave_gid = 0; wave_gid < stride; ++wave_gid) {
@@ -149,7 +149,7 @@ static int emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t*
         const int64_t gid = sub * kLanes + lane;
         chunk[lane] = fetch_chunk(codes_p, n_bytes, gid, codes_aligned);
         gap[lane] = gap_of(c_gaps.p, gid, n_gap_bytes);
-        regs[lane] = decode_chunk_regs<kMain>(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
+        regs[lane] = decode_chunk_regs(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
         all_fit = all_fit && !regs[lane].overflow;
       }
       uint32_t total = 0;
@@ -195,24 +195,6 @@ static int emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t*
   }
   memcpy(out, out_p, (size_t)n_elements * 2);
   return 0;
-}
-
-// Same data arguments as df11_decode (include/df11.h), host pointers; `grid`
-// plays gridDim.x (workgroups of eight wavefronts).  max_elems_per_sub <= 0
-// selects the worst case, as in the library.  flags: bit 0 forces the two-pass
-// route on every sub-block, bit 1 selects the compilation with the register slots
-// of the short-code launch plan.
-extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
-                                const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
-                                int n_luts, int64_t n_bytes, int64_t n_elements,
-                                int max_elems_per_sub, int grid, int codes_misalign,
-                                int out_misalign, int flags) {
-  return (flags & 2) ? emul_decode<kMainSlotsShortCodes>(luts, codes, sign_mantissa, positions, gaps, out, n_luts,
-                                                         n_bytes, n_elements, max_elems_per_sub, grid,
-                                                         codes_misalign, out_misalign, flags)
-                     : emul_decode<kMainSlots>(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes,
-                                               n_elements, max_elems_per_sub, grid, codes_misalign, out_misalign,
-                                               flags);
 }
 
 #ifdef DF11_EMUL_MAIN

@@ -29,22 +29,20 @@ def _p(a):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0, two_pass=False, short_code_slots=False):
-    """short_code_slots: the compilation of the short-code launch plan, which keeps 14
-    lookups per chunk in registers instead of 7."""
+def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0, two_pass=False):
     n = c["sign_mantissa"].size
     out = np.zeros(n, np.uint16)
     luts = np.ascontiguousarray(c["luts"])
     rc = L.df11_emul_decode(_p(luts), _p(c["encoded_exponent"]), _p(c["sign_mantissa"]),
                             _p(c["output_positions"]), _p(c["gaps"]), _p(out), luts.shape[0],
                             c["encoded_exponent"].size, n, max_elems, grid, codes_misalign, out_misalign,
-                            (1 if two_pass else 0) | (2 if short_code_slots else 0))
+                            1 if two_pass else 0)
     assert rc == 0
     return out
 
 
 def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=None, two_pass=False,
-             ok_codes=(0,), short_code_slots=False):
+             ok_codes=(0,)):
     n = c["sign_mantissa"].size
     n_bytes = c["encoded_exponent"].size
     n_blocks = -(-n_bytes // 4096)
@@ -52,7 +50,7 @@ def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=
     inp, outp = str(tmp_path / "case.bin"), str(tmp_path / "out.bin")
     with open(inp, "wb") as f:
         f.write(np.array([luts.shape[0], n_bytes, n, n_blocks, max_elems, grid, codes_misalign,
-                          out_misalign, (1 if two_pass else 0) | (2 if short_code_slots else 0)], np.int64).tobytes())
+                          out_misalign, 1 if two_pass else 0], np.int64).tobytes())
         f.write(luts.tobytes())
         f.write(c["encoded_exponent"].tobytes())
         f.write(c["sign_mantissa"].tobytes())
@@ -76,8 +74,6 @@ def test_emulated_kernel_matches_oracle(emul, oracle, kind, n):
     assert np.array_equal(got, ref)
     # worst-case staging selected by max_elems <= 0; the two-pass fall-back route on every input
     assert np.array_equal(run_emul(emul, c, max_elems=0, grid=1, two_pass=True), ref)
-    # the compilation with the register slots of the short-code plan
-    assert np.array_equal(run_emul(emul, c, max_elems=0, grid=2, short_code_slots=True), ref)
 
 
 @pytest.mark.parametrize("kind", ["normal", "zeros", "fib", "uniform256"])
@@ -157,9 +153,6 @@ def test_emulated_kernel_under_asan(emul, tmp_path, kind, n, cm, om):
         got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
                        out_misalign=om, tmp_path=tmp_path, two_pass=two_pass)
         assert np.array_equal(got, w)
-    got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
-                   out_misalign=om, tmp_path=tmp_path, short_code_slots=True)
-    assert np.array_equal(got, w)
 
 
 def test_emulated_kernel_malformed_streams_stay_in_bounds(emul, tmp_path):
@@ -367,7 +360,6 @@ def test_emulated_kernel_random_codes_and_fillings(emul, oracle, chunk):
             assert np.array_equal(ref, w), (seed, policy)
             for two_pass in (False, True):
                 assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (seed, policy, two_pass)
-            assert np.array_equal(run_emul(emul, c, short_code_slots=True), w), (seed, policy)
             ran += 1
     assert ran > 20
 
@@ -386,23 +378,6 @@ def test_emulated_kernel_every_lut_row(emul, oracle, n):
         assert np.array_equal(ref, w), policy
         for two_pass in (False, True):
             assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (policy, two_pass)
-        assert np.array_equal(run_emul(emul, c, short_code_slots=True), w), policy
-
-
-def test_emulated_kernel_short_codes_stay_in_registers(emul):
-    """Chunks of one-bit and two-bit codes need up to 16 lookups: more than the seven
-    register slots of the usual compilations, within the 14 + 2 of the short-code one.  The
-    emulation compares the register route's counts with the counting pass, and the output
-    with the original words, under both."""
-    rng = np.random.default_rng(11)
-    for p_zero in (1.0, 0.97, 0.7, 0.5):
-        n = 150_000
-        e = np.where(rng.random(n) < p_zero, 0, rng.choice([100, 101, 102], n)).astype(np.uint16)
-        sm = rng.integers(0, 256, n).astype(np.uint16)
-        w = (((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)).astype(np.uint16)
-        c = compress_product(w)
-        for short in (False, True):
-            assert np.array_equal(run_emul(emul, c, grid=2, short_code_slots=short), w), (p_zero, short)
 
 
 def test_emulated_kernel_few_elements_many_symbols(emul, oracle):
