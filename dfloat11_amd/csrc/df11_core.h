@@ -571,12 +571,19 @@ constexpr int kMaxElemsPerSub = kSubBytes * 8;           // one-bit codes
 constexpr int kGroup = 8;                                // elements per lane per write-out step
 
 // Workspace derived once per tensor: header | decode tables | sub-block positions.
+// A workspace is valid for the stream it was prepared from and for the library build
+// that prepared it: the header records the layout's number and the stream's table count
+// so that a dump of one can be told from another, but df11_decode does not read the
+// header back (that would take a device read per call).
 struct WorkspaceHeader {
   uint32_t magic;
   uint32_t n_blocks;
   uint32_t max_sub_elems;   // largest number of elements any sub-block produces
-  uint32_t reserved[13];
+  uint32_t layout;          // kWorkspaceLayout of the build that wrote it
+  uint32_t n_luts;          // rows of the stream's luts, the length row included
+  uint32_t reserved[11];
 };
+constexpr uint32_t kWorkspaceLayout = 3;            // 3: fused 16-bit LUT rows follow the tables
 constexpr uint32_t kWorkspaceMagic = 0x31314644u;   // "DF11"
 constexpr int kWsTablesOffset = 64;
 constexpr int kWsSubposOffset = kWsTablesOffset + kTablesBytes;

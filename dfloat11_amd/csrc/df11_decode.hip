@@ -104,6 +104,8 @@ __global__ __launch_bounds__(256) void build_tables_kernel(const uint8_t* __rest
     uint32_t v = 0;
     if (idx == 0) v = kWorkspaceMagic;
     if (idx == 1) v = n_blocks;
+    if (idx == 3) v = kWorkspaceLayout;
+    if (idx == 4) v = (uint32_t)n_luts;
     reinterpret_cast<uint32_t*>(ws)[idx] = v;   // max_sub_elems starts at 0
   }
 }
@@ -289,18 +291,22 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority>
+template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, bool kConstantLdsBase>
 __device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
     uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
-  // The decode kernels have no static LDS, so its dynamic LDS starts at address 0 of the
-  // workgroup's allocation (the host checks the kernel's static size before the
+  // The decode kernels have no static LDS, so their dynamic LDS starts at address 0 of the
+  // workgroup's allocation (the host checks the kernels' static size before the
   // first launch).  Spelling the base as a constant instead of the symbol of an
   // extern array lets the compiler fold it into the offset field of every LDS
   // instruction: the symbol costs one vector add per table lookup and staging
   // access.  The first kLdsSkip bytes stay unused (address 0 would read as null).
-  const LdsBytes lds = reinterpret_cast<LdsBytes>((uintptr_t)kLdsSkip);
+  // One compilation (`portable`) takes the base from the symbol all the same: it is
+  // what runs if a toolchain ever gives the other kernels LDS of its own.
+  extern __shared__ __align__(16) uint8_t dynamic_lds[];
+  const LdsBytes lds = kConstantLdsBase ? reinterpret_cast<LdsBytes>((uintptr_t)kLdsSkip)
+                                        : (LdsBytes)dynamic_lds + kLdsSkip;
   const int tid = threadIdx.x;
   const uint32_t lane = tid & 63;
   const uint32_t wave = uniform(tid >> 6);
@@ -511,20 +517,22 @@ __device__ __forceinline__ void decode_body(
 // under 38 M elements that fit its rounds better than those of `wide` (a stream that
 // small may still sit in the memory-side cache).
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
-#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd)             \
+#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd, const_lds)  \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
                                                                              waves_per_simd)))    \
   void name(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,         \
             const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,                         \
             const uint8_t* __restrict__ ws, const DecodeSizes z) {                                \
-    decode_body<prefetch, streaming, phase_priority>(codes, sign_mantissa, gaps, out, ws, z);     \
+    decode_body<prefetch, streaming, phase_priority, const_lds>(codes, sign_mantissa, gaps, out,  \
+                                                                ws, z);                           \
   }
-DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6)
-DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4)
-DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4)
-DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4)
-DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4)
-DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4)
+DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6, true)
+DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4, true)
+DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4, true)
+DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4, true)
+DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4, true)
+DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4, true)
+DF11_DECODE_KERNEL(decode_kernel_portable, 2, false, false, 6, false)   // `wide`, LDS addressed through its symbol
 #undef DF11_DECODE_KERNEL
 
 typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);
@@ -553,6 +561,7 @@ const LaunchPlan kDeepSmall{decode_kernel_deep_small, kDeepGroupsPerCu, decode_k
                             "deep/small"};
 const LaunchPlan kDeepest{decode_kernel_deepest, kDeepGroupsPerCu, decode_kernel_deepest_short, "deepest",
                           "deepest/short"};
+const LaunchPlan kPortable{decode_kernel_portable, kWideGroupsPerCu, nullptr, "portable", nullptr};
 
 // `pinned` is one of DF11_PLAN_*: anything but a plan's number leaves the choice to the rule.
 LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned = DF11_PLAN_AUTO) {
@@ -560,6 +569,7 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned =
     case DF11_PLAN_WIDE: return kWide;
     case DF11_PLAN_DEEP: return kDeep;
     case DF11_PLAN_DEEPEST: return kDeepest;
+    case DF11_PLAN_PORTABLE: return kPortable;
     default: break;
   }
   const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
@@ -593,6 +603,7 @@ bool few_rounds(int64_t n_subs, int64_t grid) {
 
 struct DeviceInfo {
   int cus = 0;
+  bool constant_lds_base = false;   // the kernels that address LDS from a constant may run
   bool ok = false;
 };
 
@@ -607,14 +618,17 @@ int device_info(DeviceInfo& info) {
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return hip_fail(e);
     // the decode kernels address their LDS from a constant base, which holds only
-    // as long as they have no static LDS of their own
+    // as long as they have no static LDS of their own; if one of them has, every
+    // stream runs the compilation that takes the base from the symbol instead
+    bool constant_base = true;
     for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deep_short, decode_kernel_deep_small,
                            decode_kernel_deepest, decode_kernel_deepest_short}) {
       hipFuncAttributes attr;
       e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(k));
       if (e != hipSuccess) return hip_fail(e);
-      if (attr.sharedSizeBytes != 0) return DF11_ERR_UNSUPPORTED;
+      if (attr.sharedSizeBytes != 0) constant_base = false;
     }
+    cache[dev].constant_lds_base = constant_base;
     cache[dev].cus = cus;
     cache[dev].ok = true;
   }
@@ -684,7 +698,8 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
   const size_t lds_bytes = (size_t)kLdsSkip + (size_t)tables_bytes(n_rows) +
                            (size_t)kWavesPerGroup * (size_t)z.stage_cap;
-  const LaunchPlan plan = plan_launch(z.n_subs, n_elements, info.cus, pinned_plan);
+  const LaunchPlan plan = plan_launch(z.n_subs, n_elements, info.cus,
+                                      info.constant_lds_base ? pinned_plan : DF11_PLAN_PORTABLE);
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, plan.groups_per_cu);
   const int64_t needed = (z.n_subs + kWavesPerGroup - 1) / kWavesPerGroup;
   if (grid > needed) grid = needed;
@@ -825,7 +840,7 @@ int df11_decode_with_plan(const uint8_t* luts, const uint8_t* encoded_exponent, 
                           int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void* workspace,
                           int32_t max_elems_per_subblock, void* stream, int32_t plan) {
   (void)output_positions;
-  if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_DEEPEST) return DF11_ERR_INVALID_ARGUMENT;
+  if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_PORTABLE) return DF11_ERR_INVALID_ARGUMENT;
   return checked_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements, workspace,
                         max_elems_per_subblock, stream, plan);
 }

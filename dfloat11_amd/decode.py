@@ -100,7 +100,7 @@ def prepare(luts, encoded_exponent, output_positions, gaps, n_elements, workspac
     return workspace, int(max_sub.value)
 
 
-PLANS = {"auto": -1, "wide": 0, "deep": 1, "deepest": 2}
+PLANS = {"auto": -1, "wide": 0, "deep": 1, "deepest": 2, "portable": 3}
 
 
 def decode(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,

@@ -212,22 +212,24 @@ _STREAM_NAMES = ('luts', 'encoded_exponent', 'sign_mantissa', 'output_positions'
 
 
 def _stream_state(module):
-    """The five stream tensors of a module as (object, in-place version) pairs: what the
-    cached launch arguments and the decode workspace were derived from.  A tensor that
-    was replaced shows as another object, one written in place (load_state_dict copies
-    into the existing buffers) as another version."""
+    """The five stream tensors of a module as (object, in-place version, address, size)
+    entries: what the cached launch arguments and the decode workspace were derived
+    from.  A tensor that was replaced shows as another object, one written in place
+    (load_state_dict copies into the existing buffers) as another version, and one
+    whose storage was rebound (`t.data = other`, `t.set_(...)`: same object, same
+    version) as another address or size."""
     state = []
     for name in _STREAM_NAMES:
         t = module._buffers.get(name)
         if t is None and name in getattr(module, 'offloaded_tensors', {}):
             t = module.offloaded_tensors[name]
-        state.append((t, t._version if t is not None else -1))
+        state.append((t, t._version, t.data_ptr(), t.numel()) if t is not None else (None, -1, 0, 0))
     return tuple(state)
 
 
 def _same_streams(module, state):
     now = _stream_state(module)
-    return all(a[0] is b[0] and a[1] == b[1] for a, b in zip(now, state))
+    return all(a[0] is b[0] and a[1:] == b[1:] for a, b in zip(now, state))
 
 
 def _workspace_for(module, device, encoded_exponent, n_elements):

@@ -97,8 +97,9 @@ int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint
 
 /*
  * df11_prepare + df11_decode in one call, with the workspace in a device array
- * that the library itself holds (DF11_STATIC_WORKSPACE_BYTES per GPU, resident
- * from the first call on that GPU until the process ends).  No counterpart in
+ * that the library itself holds (DF11_STATIC_WORKSPACE_BYTES on every GPU the
+ * library's code is loaded on, from that load until the process ends, whether
+ * this entry point is ever called or not).  No counterpart in
  * the reference: it is for callers that cannot allocate device memory or wait
  * for the device -- code under HIP graph capture, serving loops, harnesses that
  * forbid hipMalloc.  The call allocates and frees nothing, never synchronises,
@@ -110,8 +111,11 @@ int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint
  *               the format's worst case (4096), which is always safe
  * Streams of more than DF11_STATIC_MAX_STREAM_BYTES bytes of encoded_exponent
  * are rejected with DF11_ERR_CAPACITY.  All calls on one GPU share the one
- * array: calls that overlap in time on the same GPU (different streams) race;
- * the caller serialises them.  The first call on a GPU looks the array's device
+ * array: calls that overlap in time on the same GPU (different streams, or a
+ * captured graph replayed on one stream while an eager call runs on another)
+ * race and corrupt each other's output without an error; the caller orders
+ * them, with an event between streams where they differ.  The first call on a
+ * GPU looks the array's device
  * address up (hipGetSymbolAddress); make that call outside a graph capture.
  */
 #define DF11_STATIC_WORKSPACE_BYTES 4194304
@@ -128,9 +132,10 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
  * it requests sign_mantissa bytes: DF11_PLAN_WIDE, _DEEP, _DEEPEST; the two plans
  * for large streams come in further compilations that differ in how wavefront
  * priorities are set and in the cache policy of the loads, which the stream's
- * size decides in either entry point).  df11_decode picks the plan per stream from
- * its size and its elements per 512 bytes of bitstream; this entry point takes it
- * as an argument, for tests that drive every stream through every plan and for
+ * size decides in either entry point), seven kernels in all with
+ * DF11_PLAN_PORTABLE.  df11_decode picks the plan per stream from its size and
+ * its elements per 512 bytes of bitstream; this entry point takes it as an
+ * argument, for tests that drive every stream through every plan and for
  * measurements.  DF11_PLAN_AUTO behaves as df11_decode does.  The choice is local
  * to the call: nothing in the library remembers it.  No counterpart in the
  * reference; every plan decodes every stream to the same bits.
@@ -139,6 +144,11 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
 #define DF11_PLAN_WIDE 0
 #define DF11_PLAN_DEEP 1
 #define DF11_PLAN_DEEPEST 2
+/* `wide` with workgroup memory addressed through its symbol instead of from a constant:
+ * what every stream runs, whatever plan is asked for, if a toolchain gives the other
+ * kernels workgroup memory of its own (checked once per device); about 13 % more vector
+ * instructions. */
+#define DF11_PLAN_PORTABLE 3
 int df11_decode_with_plan(const uint8_t *luts, const uint8_t *encoded_exponent,
                           const uint8_t *sign_mantissa, const uint32_t *output_positions,
                           const uint8_t *gaps, uint16_t *outputs, int32_t n_luts, int64_t n_bytes,

@@ -83,6 +83,8 @@ extern "C" int df11_emul_prepare(const uint8_t* luts, const uint8_t* codes, cons
   h.magic = kWorkspaceMagic;
   h.n_blocks = (uint32_t)n_blocks;
   h.max_sub_elems = max_sub;
+  h.layout = kWorkspaceLayout;
+  h.n_luts = (uint32_t)n_luts;
   memcpy(ws, &h, sizeof h);
   return (int)max_sub;
 }

@@ -78,10 +78,10 @@ def test_plan_argument_is_validated_before_anything_else():
     no GPU and no valid pointers are needed to see it.  No call changes what a later call does:
     the library keeps no launch state."""
     hip = _native.hip_lib()
-    for plan in (3, -2, 100):
+    for plan in (4, -2, 100):
         assert hip.df11_decode_with_plan(None, None, None, None, None, None, 2, 16, 16, None, 0, None, plan) == -1
     # an empty stream is a successful no-op under every plan
-    for plan in (-1, 0, 1, 2):
+    for plan in (-1, 0, 1, 2, 3):
         assert hip.df11_decode_with_plan(None, None, None, None, None, None, 2, 0, 0, None, 0, None, plan) == 0
 
 

@@ -316,3 +316,40 @@ def test_streams_rewritten_in_place_are_decoded_anew(tmp_path):
         want = ref_b.to(DEV)(ids)
         assert torch.equal(model(ids), want)
         assert torch.equal(model(ids), want)
+
+
+def test_streams_rebound_to_other_storage_are_decoded_anew(tmp_path):
+    """`buffer.data = other` keeps the tensor object and its version counter and points it
+    at other memory: the cached launch arguments hold the old addresses and must not be
+    used again, nor the workspace derived from the old contents."""
+    print("case api streams rebound to other storage", flush=True)
+    from safetensors.torch import load_file
+    M._prefetcher.reset()
+    a, b = make_model(12), make_model(12)
+    with torch.no_grad():
+        for p in b.parameters():
+            if p.dim() > 1:
+                p.copy_(p.flatten().flip(0).view_as(p))
+    ref_b = make_model(12)
+    ref_b.load_state_dict(b.state_dict())
+    compress_model(a, PATTERNS, str(tmp_path / "a"), check_correctness=False)
+    compress_model(b, PATTERNS, str(tmp_path / "b"), check_correctness=False)
+    model = DFloat11Model.from_pretrained(str(tmp_path / "a"), device=DEV, bfloat16_model=make_model(9))
+    ids = torch.randint(0, 97, (2, 8), device=DEV)
+    with torch.no_grad():
+        assert torch.equal(model(ids), _reference_logits(12, ids))
+        assert torch.equal(model(ids), _reference_logits(12, ids))      # launch arguments bound by now
+        state_b = load_file(str(tmp_path / "b" / "model.safetensors"))
+        keep = []                                                       # the old storages stay alive: a stale address would still decode
+        for name, module in model.named_modules():
+            for key in ("luts", "encoded_exponent", "sign_mantissa", "output_positions", "gaps"):
+                full = f"{name}.{key}" if name else key
+                if full in state_b and key in module._buffers:
+                    buf = module._buffers[key]
+                    keep.append(buf.data)
+                    version = buf._version
+                    buf.data = state_b[full].to(DEV)
+                    assert buf._version == version
+        want = ref_b.to(DEV)(ids)
+        assert torch.equal(model(ids), want)
+        assert torch.equal(model(ids), want)

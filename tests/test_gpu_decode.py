@@ -58,11 +58,12 @@ def test_gpu_matches_oracle(oracle, kind, n):
     assert np.array_equal(got, w)
 
 
-@pytest.mark.parametrize("plan", [0, 1, 2], ids=["wide", "deep", "deepest"])
+@pytest.mark.parametrize("plan", [0, 1, 2, 3], ids=["wide", "deep", "deepest", "portable"])
 def test_gpu_every_launch_plan_matches_oracle(oracle, plan):
     """The plans differ in resident workgroups and in how many groups of sign|mantissa
-    bytes are requested early; the automatic choice sends small streams to one of them
-    only.  Through df11_decode_with_plan each plan decodes every kind, ragged sizes,
+    bytes are requested early (`portable` is `wide` with LDS addressed through its symbol,
+    the compilation kept for a toolchain on which the constant LDS base of the others does
+    not hold); the automatic choice sends small streams to one of them only.  Through df11_decode_with_plan each plan decodes every kind, ragged sizes,
     unaligned buffers and the worst-case staging to the oracle's bits."""
     for kind in KINDS:
         for n in (1, 511, 4097, 70_001, 300_000):
