@@ -56,6 +56,8 @@ def hip_lib():
         L.df11_decode_static_workspace.restype = _i32
         L.df11_decode_with_plan.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp, _i32]
         L.df11_decode_with_plan.restype = _i32
+        L.df11_decode_rows.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _i32, _vp, _vp, _i64, _i64]
+        L.df11_decode_rows.restype = _i32
         L.df11_launch_plan_name.argtypes = [_i64, _i64, _i32]
         L.df11_launch_plan_name.restype = ctypes.c_char_p
         _hip = L

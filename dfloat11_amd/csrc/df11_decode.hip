@@ -291,11 +291,42 @@ __device__ __forceinline__ SubInputs fetch_sub(const uint8_t* __restrict__ codes
   return in;
 }
 
-template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, bool kConstantLdsBase>
+// Rows of a matrix to decode (decode_kernel_rows): the elements
+// [id * row_elements, (id + 1) * row_elements) of the stream's output for each id.
+struct RowsArgs {
+  const int64_t* ids;
+  int64_t n_ids;
+  int64_t row_elements;
+};
+
+// Index of the sub-block that holds output element `start` (< n_elements): the last
+// entry of the ascending `subpos` (n_entries of them, the first is 0) that is <= start.
+// The 64 lanes probe 64 evenly spaced entries at a time, so a search over 2^24 entries
+// takes four dependent loads.  The result is wavefront-uniform.
+__device__ __forceinline__ uint32_t find_sub(const uint32_t* __restrict__ subpos, uint32_t n_entries,
+                                             uint32_t start, uint32_t lane) {
+  uint32_t lo = 0, hi = n_entries;   // the answer lies in [lo, hi) and subpos[lo] <= start
+  while (hi - lo > (uint32_t)kLanes) {
+    const uint32_t step = (hi - lo + (uint32_t)kLanes - 1u) / (uint32_t)kLanes;
+    const uint32_t probe = lo + lane * step;
+    const bool le = probe < hi && subpos[probe] <= start;
+    // ascending entries: the lanes that say yes are a run from lane 0, which is one of them
+    // (at least one is assumed, so that entries that do not ascend cannot lead anywhere odd)
+    const uint32_t k = max(1u, (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le)));
+    lo += (k - 1u) * step;
+    hi = min(hi, lo + step);
+  }
+  const uint32_t probe = lo + lane;
+  const bool le = probe < hi && subpos[probe] <= start;
+  return lo + max(1u, (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le))) - 1u;
+}
+
+template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, bool kConstantLdsBase, bool kRows = false>
 __device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
-    uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z) {
+    uint16_t* __restrict__ out, const uint8_t* __restrict__ ws, const DecodeSizes z,
+    const RowsArgs rows = RowsArgs{}) {
   // The decode kernels have no static LDS, so their dynamic LDS starts at address 0 of the
   // workgroup's allocation (the host checks the kernels' static size before the
   // first launch).  Spelling the base as a constant instead of the symbol of an
@@ -325,8 +356,8 @@ __device__ __forceinline__ void decode_body(
   const uint32_t vzero = opaque_vector_zero();
   // The first sub-block's inputs are requested before the tables are copied, so
   // that their latency overlaps with that of the copy.
-  SubInputs cur{};
-  if (sub < z.n_subs) cur = fetch_sub<kStreaming>(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
+  SubInputs held{};
+  if (!kRows && sub < z.n_subs) held = fetch_sub<kStreaming>(codes, gaps, subpos, z, sub, lane, gap_byte, vzero);
   {
     const uint4* src = reinterpret_cast<const uint4*>(ws + kWsTablesOffset);
     for (int i = tid; i < tables_bytes(n_rows) / 16; i += kThreads) lds_store<uint4>(lds_tables + 16 * i, src[i]);
@@ -340,8 +371,8 @@ __device__ __forceinline__ void decode_body(
   const Rows l{lds_tables + kRowsOffset};
   const bool vec_ok = z.vec_ok != 0;
   const int64_t stride = (int64_t)gridDim.x * kWavesPerGroup;
-  if (sub >= z.n_subs) return;
-  claim(cur.d0, cur.d1, cur.d2, cur.gap_raw, cur.base, cur.end_hint);   // see the claim inside the loop
+  if (!kRows && sub >= z.n_subs) return;
+  claim(held.d0, held.d1, held.d2, held.gap_raw, held.base, held.end_hint);   // see the claim inside the step
 
   // The instruction arbiter prefers the oldest wavefront of a SIMD, so with equal
   // shares of work the wavefronts launched first would finish well before the
@@ -355,7 +386,9 @@ __device__ __forceinline__ void decode_body(
   // sub-block's inputs, so that stores and loads are issued as soon as they can be
   // and the decodes of the other wavefronts fill the gaps.
   uint32_t turn = __builtin_amdgcn_s_getreg((3 << 11) | 4);   // HW_ID.WAVE_ID, the slot on the SIMD
-  for (; sub < z.n_subs; sub += stride) {
+  // One sub-block, whose inputs `cur` holds; returns the inputs of sub-block `next_sub`,
+  // requested on the way if `fetch_next` says that it exists.
+  auto step = [&](const SubInputs& cur, bool fetch_next, int64_t next_sub) __attribute__((always_inline)) -> SubInputs {
     if (!kPhasePriority) {
       switch (turn++ & 3u) {   // s_setprio takes an immediate
         case 0: __builtin_amdgcn_s_setprio(0); break;
@@ -366,9 +399,8 @@ __device__ __forceinline__ void decode_body(
     }
     // ---- requests whose latency the two decode passes hide: the next
     // sub-block's inputs and this one's sign|mantissa bytes
-    const int64_t next_sub = sub + stride;
     SubInputs nxt = cur;
-    if (next_sub < z.n_subs) nxt = fetch_sub<kStreaming>(codes, gaps, subpos, z, next_sub, lane, gap_byte, vzero);
+    if (fetch_next) nxt = fetch_sub<kStreaming>(codes, gaps, subpos, z, next_sub, lane, gap_byte, vzero);
 
     const uint32_t base = uniform(cur.base);
     const uint32_t a0 = base & ~(uint32_t)(kGroup - 1);
@@ -489,7 +521,34 @@ __device__ __forceinline__ void decode_body(
     for (uint32_t i = lane * 8u; i < stage_used(p); i += kLanes * 8u) lds_store<U32x2>(stage + i, U32x2{0, 0});
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    cur = nxt;
+    return nxt;
+  };
+
+  if (kRows) {
+    // Workgroup i takes ids i, i + grid, ...; its eight wavefronts take the sub-blocks
+    // that overlap the id's elements in turn.  Each sub-block is written out whole, so
+    // the elements next to a row, up to a sub-block's worth on either side, are decoded
+    // with it (to the same values any other decode of them writes).
+    const uint32_t n_entries = (uint32_t)(z.n_blocks * kSubsPerBlock + 1);
+    const int64_t n_rows_total = rows.row_elements > 0 ? z.n_elements / rows.row_elements : 0;
+    for (int64_t i = blockIdx.x; i < rows.n_ids; i += gridDim.x) {
+      const int64_t id = rows.ids[i];                         // uniform
+      if (id < 0 || id >= n_rows_total) continue;             // ids outside the matrix select nothing
+      const int64_t first = id * rows.row_elements;
+      const int64_t end = first + rows.row_elements;
+      const uint32_t s0 = uniform(find_sub(subpos, n_entries, (uint32_t)first, lane));
+      for (int64_t s = (int64_t)s0 + wave; s < z.n_subs; s += kWavesPerGroup) {
+        SubInputs in = fetch_sub<kStreaming>(codes, gaps, subpos, z, s, lane, gap_byte, vzero);
+        if ((int64_t)uniform(in.base) >= end) break;          // starts past the row
+        claim(in.d0, in.d1, in.d2, in.gap_raw, in.base, in.end_hint);
+        step(in, false, 0);
+      }
+    }
+    return;
+  }
+  for (; sub < z.n_subs; sub += stride) {
+    const int64_t next_sub = sub + stride;
+    held = step(held, next_sub < z.n_subs, next_sub);
   }
 }
 
@@ -534,6 +593,16 @@ DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4, true)
 DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4, true)
 DF11_DECODE_KERNEL(decode_kernel_portable, 2, false, false, 6, false)   // `wide`, LDS addressed through its symbol
 #undef DF11_DECODE_KERNEL
+
+// Decodes only the sub-blocks that hold given rows of the output matrix (an embedding
+// looks up a few rows of a table whose stream holds them all): `wide` settings, wavefront
+// priorities by phase, work taken per id instead of per sub-block.
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6)))
+void decode_kernel_rows(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,
+                        const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,
+                        const uint8_t* __restrict__ ws, const DecodeSizes z, const RowsArgs rows) {
+  decode_body<2, false, true, true, true>(codes, sign_mantissa, gaps, out, ws, z, rows);
+}
 
 typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);
 struct LaunchPlan {
@@ -621,10 +690,14 @@ int device_info(DeviceInfo& info) {
     // as long as they have no static LDS of their own; if one of them has, every
     // stream runs the compilation that takes the base from the symbol instead
     bool constant_base = true;
-    for (DecodeKernel k : {decode_kernel_wide, decode_kernel_deep, decode_kernel_deep_short, decode_kernel_deep_small,
-                           decode_kernel_deepest, decode_kernel_deepest_short}) {
+    for (const void* k : {reinterpret_cast<const void*>(decode_kernel_wide), reinterpret_cast<const void*>(decode_kernel_deep),
+                          reinterpret_cast<const void*>(decode_kernel_deep_short),
+                          reinterpret_cast<const void*>(decode_kernel_deep_small),
+                          reinterpret_cast<const void*>(decode_kernel_deepest),
+                          reinterpret_cast<const void*>(decode_kernel_deepest_short),
+                          reinterpret_cast<const void*>(decode_kernel_rows)}) {
       hipFuncAttributes attr;
-      e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(k));
+      e = hipFuncGetAttributes(&attr, k);
       if (e != hipSuccess) return hip_fail(e);
       if (attr.sharedSizeBytes != 0) constant_base = false;
     }
@@ -675,12 +748,9 @@ int enqueue_prepare(const uint8_t* luts, const uint8_t* encoded_exponent, const 
   return DF11_OK;
 }
 
-// Enqueues the decode of one stream whose workspace `ws` is (or will be, in
-// stream order) filled.
-int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
-                   const uint8_t* gaps, uint16_t* outputs, int32_t n_luts, int64_t n_bytes,
-                   int64_t n_elements, const uint8_t* ws, int32_t max_elems_per_subblock,
-                   const DeviceInfo& info, hipStream_t s, int pinned_plan = DF11_PLAN_AUTO) {
+// Sizes and alignment facts of a stream as the decode kernels take them.
+DecodeSizes decode_sizes(const uint8_t* encoded_exponent, const uint8_t* sign_mantissa, const uint16_t* outputs,
+                         int32_t n_luts, int64_t n_bytes, int64_t n_elements, int32_t max_elems_per_subblock) {
   if (max_elems_per_subblock <= 0 || max_elems_per_subblock > kMaxElemsPerSub)
     max_elems_per_subblock = kMaxElemsPerSub;
   DecodeSizes z;
@@ -693,11 +763,24 @@ int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const u
   z.codes_aligned = (reinterpret_cast<uintptr_t>(encoded_exponent) & 7) == 0;
   z.vec_ok = (reinterpret_cast<uintptr_t>(sign_mantissa) & 7) == 0 &&
              (reinterpret_cast<uintptr_t>(outputs) & 15) == 0;
+  return z;
+}
 
-  // LDS: tables, the fused LUT rows that exist, one staging area per wavefront
-  const int n_rows = n_luts - 1 < kMaxDecodeRows ? n_luts - 1 : kMaxDecodeRows;
-  const size_t lds_bytes = (size_t)kLdsSkip + (size_t)tables_bytes(n_rows) +
-                           (size_t)kWavesPerGroup * (size_t)z.stage_cap;
+// LDS of one workgroup: tables, the fused LUT rows that exist, one staging area per wavefront.
+size_t decode_lds_bytes(const DecodeSizes& z) {
+  const int n_rows = z.n_luts - 1 < kMaxDecodeRows ? z.n_luts - 1 : kMaxDecodeRows;
+  return (size_t)kLdsSkip + (size_t)tables_bytes(n_rows) + (size_t)kWavesPerGroup * (size_t)z.stage_cap;
+}
+
+// Enqueues the decode of one stream whose workspace `ws` is (or will be, in
+// stream order) filled.
+int enqueue_decode(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
+                   const uint8_t* gaps, uint16_t* outputs, int32_t n_luts, int64_t n_bytes,
+                   int64_t n_elements, const uint8_t* ws, int32_t max_elems_per_subblock,
+                   const DeviceInfo& info, hipStream_t s, int pinned_plan = DF11_PLAN_AUTO) {
+  const DecodeSizes z = decode_sizes(encoded_exponent, sign_mantissa, outputs, n_luts, n_bytes, n_elements,
+                                     max_elems_per_subblock);
+  const size_t lds_bytes = decode_lds_bytes(z);
   const LaunchPlan plan = plan_launch(z.n_subs, n_elements, info.cus,
                                       info.constant_lds_base ? pinned_plan : DF11_PLAN_PORTABLE);
   int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, plan.groups_per_cu);
@@ -746,7 +829,7 @@ int scratch_of_current_device(uint8_t** out) {
 
 extern "C" {
 
-int df11_version(void) { return 4; }
+int df11_version(void) { return 5; }
 
 const char* df11_error_string(int code) {
   switch (code) {
@@ -843,6 +926,39 @@ int df11_decode_with_plan(const uint8_t* luts, const uint8_t* encoded_exponent, 
   if (plan < DF11_PLAN_AUTO || plan > DF11_PLAN_PORTABLE) return DF11_ERR_INVALID_ARGUMENT;
   return checked_decode(luts, encoded_exponent, sign_mantissa, gaps, outputs, n_luts, n_bytes, n_elements, workspace,
                         max_elems_per_subblock, stream, plan);
+}
+
+int df11_decode_rows(const uint8_t* luts, const uint8_t* encoded_exponent, const uint8_t* sign_mantissa,
+                     const uint32_t* output_positions, const uint8_t* gaps, uint16_t* outputs,
+                     int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void* workspace,
+                     int32_t max_elems_per_subblock, void* stream, const int64_t* row_ids, int64_t n_ids,
+                     int64_t row_elements) {
+  (void)output_positions;
+  if (n_bytes < 0 || n_elements < 0 || n_luts < 2 || n_ids < 0 || row_elements <= 0) return DF11_ERR_INVALID_ARGUMENT;
+  if (n_bytes == 0 || n_elements == 0 || n_ids == 0) return DF11_OK;
+  if (!luts || !encoded_exponent || !sign_mantissa || !gaps || !outputs || !workspace || !row_ids)
+    return DF11_ERR_INVALID_ARGUMENT;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 15) || (reinterpret_cast<uintptr_t>(outputs) & 1) ||
+      (reinterpret_cast<uintptr_t>(row_ids) & 7))
+    return DF11_ERR_INVALID_ARGUMENT;
+  if (n_elements >= ((int64_t)1 << 32)) return DF11_ERR_UNSUPPORTED;   // positions are u32
+  DeviceInfo info;
+  if (int rc = device_info(info)) return rc;
+  if (!info.constant_lds_base) return DF11_ERR_UNSUPPORTED;   // callers decode the whole stream instead
+  const DecodeSizes z = decode_sizes(encoded_exponent, sign_mantissa, outputs, n_luts, n_bytes, n_elements,
+                                     max_elems_per_subblock);
+  const size_t lds_bytes = decode_lds_bytes(z);
+  int64_t grid = (int64_t)info.cus * groups_per_cu(lds_bytes, kWideGroupsPerCu);
+  if (grid > n_ids) grid = n_ids;
+  RowsArgs rows;
+  rows.ids = row_ids;
+  rows.n_ids = n_ids;
+  rows.row_elements = row_elements;
+  hipLaunchKernelGGL(decode_kernel_rows, dim3((unsigned)grid), dim3(kThreads), lds_bytes,
+                     static_cast<hipStream_t>(stream), encoded_exponent, sign_mantissa, gaps, outputs,
+                     static_cast<const uint8_t*>(workspace), z, rows);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? DF11_OK : hip_fail(e);
 }
 
 int df11_decode_static_workspace(const uint8_t* luts, const uint8_t* encoded_exponent,

@@ -149,6 +149,30 @@ def bind(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, wor
             luts.shape[0], n_bytes, n_elements, workspace.data_ptr(), int(max_elems_per_subblock))
 
 
+def decode_rows(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,
+                max_elems_per_subblock, row_ids, row_elements):
+    """Decode only the rows `row_ids` (int64 device tensor) of the stream's output, taken as a
+    matrix of row_elements elements per row, into their places in `out` (full size)."""
+    bound = bind(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,
+                 max_elems_per_subblock)
+    launch_rows(bound, out.device, row_ids, row_elements)
+    return out
+
+
+def launch_rows(bound, device, row_ids, row_elements):
+    """df11_decode_rows with arguments from bind(): decodes the rows of the output matrix
+    (row_elements elements each) that the int64 device tensor `row_ids` names, into
+    their places in the bound output buffer; the rest of the buffer is left as it is."""
+    if row_ids.dtype != torch.int64 or row_ids.device != device or not row_ids.is_contiguous():
+        raise _native.DF11Error("row_ids must be a contiguous int64 tensor on the stream's device")
+    lib = _native.hip_lib()
+    with torch.cuda.device(device):
+        rc = lib.df11_decode_rows(*bound, torch.cuda.current_stream(device).cuda_stream,
+                                  row_ids.data_ptr(), row_ids.numel(), int(row_elements))
+    if rc:
+        _native.check(rc, "df11_decode_rows")
+
+
 def launch(bound, device):
     """df11_decode with arguments from bind(), on the current stream of `device`."""
     lib = _native.hip_lib()

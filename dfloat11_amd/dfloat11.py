@@ -252,6 +252,25 @@ def _workspace_for(module, device, encoded_exponent, n_elements):
     return module._df11_workspace, module._df11_max_sub
 
 
+# An embedding's forward reads the rows it looks up and nothing else, so its hook decodes
+# only those (df11_decode_rows) once the module's launch arguments are bound, i.e. from
+# its second call on; set to False to decode the whole table before every lookup, as the
+# reference does (reference: dfloat11.py:153-157).
+EMBEDDING_ROW_DECODE = True
+
+
+def _looked_up_rows(module, inputs, device):
+    """The row numbers an nn.Embedding is about to look up, as a contiguous int64 tensor on
+    `device`, if decoding just those rows is the cheaper call; else None."""
+    if not EMBEDDING_ROW_DECODE or not inputs or not isinstance(inputs[0], torch.Tensor):
+        return None
+    ids = inputs[0]
+    if ids.dtype != torch.int64 or ids.device != device or ids.numel() == 0 \
+            or ids.numel() * 8 > module.num_embeddings:
+        return None
+    return ids if ids.is_contiguous() else ids.contiguous()
+
+
 def get_hook(threads_per_block, bytes_per_thread):
     """Forward-pre-hook factory (reference: dfloat11.py:103-176).  The hook reads
     the module attributes luts, encoded_exponent, sign_mantissa, output_positions,
@@ -263,7 +282,7 @@ def get_hook(threads_per_block, bytes_per_thread):
             f'DF11 streams with threads_per_block={threads_per_block}, bytes_per_thread={bytes_per_thread} '
             'are not supported (only 512 x 8)')
 
-    def decode_hook(module, _):
+    def decode_hook(module, inputs):
         device = module.luts.device
         if device.type != 'cuda':
             raise RuntimeError(
@@ -277,7 +296,11 @@ def get_hook(threads_per_block, bytes_per_thread):
         if plan is not None and plan[0] is TensorManager._tensors.get(device) \
                 and _same_streams(module, plan[1]) \
                 and all(owner.__dict__.get('weight') is view for owner, view in plan[3]):
-            _decode.launch(plan[2], device)
+            row_ids = _looked_up_rows(module, inputs, device) if plan[4] else None
+            if row_ids is not None:
+                _decode.launch_rows(plan[2], device, row_ids, plan[4])
+            else:
+                _decode.launch(plan[2], device)
             return
 
         # Each of the two large streams comes from the prefetcher when the module holds it in
@@ -313,8 +336,9 @@ def get_hook(threads_per_block, bytes_per_thread):
         if parity is not None:
             _prefetcher.after_decode(module, device, parity)
         else:
+            row_elements = module.embedding_dim if isinstance(module, nn.Embedding) else 0
             object.__setattr__(module, '_df11_plan', (TensorManager._tensors.get(device), _stream_state(module),
-                                                      bound, injected))
+                                                      bound, injected, row_elements))
 
     return decode_hook
 

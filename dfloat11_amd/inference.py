@@ -138,12 +138,24 @@ def _random_prompts(model, batch_size, prompt_len, seed, device):
     return {"input_ids": ids, "attention_mask": torch.ones_like(ids)}
 
 
-def compare_synthetic(shape, batch_sizes, num_tokens, prompt_len=64, seed=42, device="cuda:0", layers=None):
+def _median_run(model, inputs, num_tokens, repeats):
+    """timed_generate `repeats` times; the run of median latency and its output."""
+    runs = [timed_generate(model, inputs, num_tokens, False) for _ in range(max(1, repeats))]
+    runs.sort(key=lambda r: r[1]["latency_s"])
+    out, stats = runs[len(runs) // 2]
+    stats["timed_runs"] = len(runs)
+    return out, stats
+
+
+def compare_synthetic(shape, batch_sizes, num_tokens, prompt_len=64, seed=42, device="cuda:0", layers=None,
+                      repeats=1):
     """Builds the named architecture once with random-init BF16 weights, generates
     greedily at every batch size, compresses the model in memory and generates again
     from the same prompts.  Returns one report per batch size with the fields of the
     reference's benchmark for both models (reference: inference.py:62-97), their
-    ratio, and whether logits and tokens are identical."""
+    ratio, and whether logits and tokens are identical.  With repeats > 1 every figure is
+    the run of median latency out of that many (generation speed of the eager model varies
+    by several per cent from run to run on the same box)."""
     import torch
     device = torch.device(device)
     model = build_synthetic(shape, device, seed, layers)
@@ -154,7 +166,7 @@ def compare_synthetic(shape, batch_sizes, num_tokens, prompt_len=64, seed=42, de
         with torch.no_grad():
             ref_logits = model(**inputs, use_cache=False).logits
         timed_generate(model, inputs, min(8, num_tokens), False)           # warm-up
-        ref_out, stats = timed_generate(model, inputs, num_tokens, False)
+        ref_out, stats = _median_run(model, inputs, num_tokens, repeats)
         reports.append({"batch_size": b, "num_tokens": num_tokens, "model": name, "prompt_len": prompt_len,
                         "bf16": stats})
         kept.append((inputs, ref_logits.cpu(), ref_out))
@@ -170,7 +182,7 @@ def compare_synthetic(shape, batch_sizes, num_tokens, prompt_len=64, seed=42, de
         with torch.no_grad():
             logits = model(**inputs, use_cache=False).logits
         timed_generate(model, inputs, min(8, num_tokens), False)
-        out, stats = timed_generate(model, inputs, num_tokens, False)
+        out, stats = _median_run(model, inputs, num_tokens, repeats)
         report["df11"] = stats
         report["logits_bit_identical"] = bool(torch.equal(logits.cpu(), ref_logits))
         report["tokens_identical"] = bool(torch.equal(out, ref_out))

@@ -39,9 +39,10 @@ extern "C" {
 #define DF11_SUBBLOCK_BYTES 512
 #define DF11_MAX_ELEMS_PER_SUBBLOCK 4096
 
-/* Version of this interface: 4 = df11_decode_with_plan replaces the process-wide
- * df11_force_launch_plan, df11_calibration_copy removed (3 = df11_decode_static_workspace
- * and df11_launch_plan_name added, workspace holds fused LUT rows). */
+/* Version of this interface: 5 = df11_decode_rows and DF11_PLAN_PORTABLE added
+ * (4 = df11_decode_with_plan replaces the process-wide df11_force_launch_plan,
+ * df11_calibration_copy removed; 3 = df11_decode_static_workspace and
+ * df11_launch_plan_name added, workspace holds fused LUT rows). */
 int df11_version(void);
 const char *df11_error_string(int code);
 
@@ -94,6 +95,29 @@ int df11_decode(const uint8_t *luts, const uint8_t *encoded_exponent, const uint
                 const uint32_t *output_positions, const uint8_t *gaps, uint16_t *outputs,
                 int32_t n_luts, int64_t n_bytes, int64_t n_elements,
                 const void *workspace, int32_t max_elems_per_subblock, void *stream);
+
+/*
+ * df11_decode for some rows of the output only: the stream decodes to a matrix of
+ * row_elements elements per row, and only the 512-byte pieces of bitstream that hold
+ * elements of rows row_ids[0 .. n_ids) are decoded, into the same places of `outputs`
+ * (the full-size buffer) that df11_decode writes them to.  Every such piece is written
+ * out whole, so up to a piece's worth of elements before and after a row are decoded
+ * with it; every other element of `outputs` is left as it was.  For an embedding,
+ * whose forward pass reads the rows it looks up and nothing else (reference:
+ * dfloat11.py:155-157 decodes the whole table before every lookup).
+ *   row_ids     DEVICE pointer to n_ids row numbers (int64, 8-byte aligned), read by
+ *               the kernel in stream order: the caller need not know them.  Numbers
+ *               outside the matrix select nothing; repeated ones cost repeated work.
+ * Other arguments and return codes as for df11_decode; DF11_ERR_UNSUPPORTED where only
+ * DF11_PLAN_PORTABLE can run (decode the whole stream there).  The work is
+ * proportional to n_ids, with a search per id on top: beyond a quarter of the rows or
+ * so, df11_decode is the faster call.
+ */
+int df11_decode_rows(const uint8_t *luts, const uint8_t *encoded_exponent, const uint8_t *sign_mantissa,
+                     const uint32_t *output_positions, const uint8_t *gaps, uint16_t *outputs,
+                     int32_t n_luts, int64_t n_bytes, int64_t n_elements, const void *workspace,
+                     int32_t max_elems_per_subblock, void *stream, const int64_t *row_ids,
+                     int64_t n_ids, int64_t row_elements);
 
 /*
  * df11_prepare + df11_decode in one call, with the workspace in a device array

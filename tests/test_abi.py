@@ -25,7 +25,7 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_error_strings():
     hip = _native.hip_lib()
-    assert hip.df11_version() == 4
+    assert hip.df11_version() == 5
     assert hip.df11_error_string(0) == b"ok"
     assert hip.df11_error_string(-1) == b"invalid argument"
     # header + tables + 17 fused LUT rows + (8 sub-blocks per 4096-byte block + 1) positions, rounded to 16
@@ -83,6 +83,16 @@ def test_plan_argument_is_validated_before_anything_else():
     # an empty stream is a successful no-op under every plan
     for plan in (-1, 0, 1, 2, 3):
         assert hip.df11_decode_with_plan(None, None, None, None, None, None, 2, 0, 0, None, 0, None, plan) == 0
+
+
+def test_row_decode_arguments_are_validated_without_a_gpu():
+    hip = _native.hip_lib()
+    rows = hip.df11_decode_rows
+    assert rows(None, None, None, None, None, None, 4, 100, 100, None, 0, None, None, 3, 10) == -1     # null pointers
+    assert rows(None, None, None, None, None, None, 4, 100, 100, None, 0, None, None, 3, 0) == -1      # no row length
+    assert rows(None, None, None, None, None, None, 4, 100, 100, None, 0, None, None, -1, 10) == -1
+    assert rows(None, None, None, None, None, None, 4, 100, 100, None, 0, None, None, 0, 10) == 0      # no rows asked for
+    assert rows(None, None, None, None, None, None, 4, 0, 0, None, 0, None, None, 3, 10) == 0          # empty stream
 
 
 def test_launch_plan_follows_stream_size_and_code_lengths():

@@ -353,3 +353,60 @@ def test_streams_rebound_to_other_storage_are_decoded_anew(tmp_path):
         want = ref_b.to(DEV)(ids)
         assert torch.equal(model(ids), want)
         assert torch.equal(model(ids), want)
+
+
+def test_embedding_decodes_only_the_rows_it_looks_up(tmp_path):
+    """From its second call on, a compressed nn.Embedding decodes just the rows of its input
+    ids: outputs stay bit-identical to the BF16 model's for changing ids (repeated, first and
+    last row, non-contiguous views), rows that were not asked for are left as they were in the
+    shared buffer, and with the switch off the whole table is decoded as before."""
+    print("case api embedding row decode", flush=True)
+    import torch.nn as nn
+    M._prefetcher.reset()
+    M.TensorManager.clear()
+    torch.manual_seed(3)
+    vocab, dim = 5000, 192
+
+    class Holder(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.embed = nn.Embedding(vocab, dim).to(torch.bfloat16)
+
+        def forward(self, ids):
+            return self.embed(ids)
+
+    source = Holder()
+    ref_weight = source.embed.weight.detach().clone().to(DEV)
+    compress_model(source, {r"embed": []}, str(tmp_path / "e"), check_correctness=False)
+    shell = Holder()
+    model = DFloat11Model.from_pretrained(str(tmp_path / "e"), device=DEV, bfloat16_model=shell)
+    g = torch.Generator().manual_seed(1)
+    with torch.no_grad():
+        ids = torch.randint(0, vocab, (4, 16), generator=g).to(DEV)
+        assert torch.equal(model(ids), ref_weight[ids])                 # first call: whole table, arguments bound
+        buf = M.TensorManager._tensors[torch.device(DEV)]
+        for shape in ((1, 1), (3, 7), (4, 16)):
+            buf.view(torch.int16).fill_(0x1234)                         # what another module's decode leaves behind
+            ids = torch.randint(0, vocab, shape, generator=g).to(DEV)
+            ids.view(-1)[0] = 0
+            ids.view(-1)[-1] = vocab - 1
+            assert torch.equal(model(ids), ref_weight[ids]), shape
+            table = model.embed.weight
+            untouched = (table.view(torch.int16) == 0x1234).all(dim=1)
+            assert int(untouched.sum()) > vocab // 2                    # only the neighbourhood of the rows was decoded
+            assert not untouched[ids.view(-1)].any()
+        wide = torch.randint(0, vocab, (6, 40), generator=g).to(DEV)
+        narrow = wide[:, -1:]                                           # non-contiguous view, as generate() passes
+        assert not narrow.is_contiguous()
+        assert torch.equal(model(narrow), ref_weight[narrow])
+        many = torch.randint(0, vocab, (40, 64), generator=g).to(DEV)   # more than an eighth of the rows: whole table
+        buf.view(torch.int16).fill_(0x1234)
+        assert torch.equal(model(many), ref_weight[many])
+        assert torch.equal(model.embed.weight, ref_weight)
+        M.EMBEDDING_ROW_DECODE = False
+        try:
+            buf.view(torch.int16).fill_(0x1234)
+            assert torch.equal(model(ids), ref_weight[ids])
+            assert torch.equal(model.embed.weight, ref_weight)
+        finally:
+            M.EMBEDDING_ROW_DECODE = True

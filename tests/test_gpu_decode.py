@@ -396,3 +396,48 @@ def test_gpu_plain_c_caller_round_trip(n):
     res = subprocess.run([exe, str(n)], capture_output=True, text=True, timeout=100)
     assert res.returncode == 0, res.stdout + res.stderr
     assert "mismatches 0" in res.stdout
+
+
+@pytest.mark.parametrize("kind,n_rows,row_elements", [("normal", 3000, 512), ("normal", 200, 4096), ("zeros", 4000, 256),
+                                                     ("uniform256", 1500, 320), ("fib", 5000, 64),
+                                                     ("laplace", 7, 100_003), ("outliers", 100_000, 3)])
+def test_gpu_rows_match_full_decode(oracle, kind, n_rows, row_elements):
+    """df11_decode_rows writes the requested rows exactly as df11_decode (and the oracle)
+    does, writes nothing but correct values anywhere else, and leaves elements that are far
+    from every requested row alone.  Row numbers repeat, come unsorted, include the first
+    and the last row and numbers outside the matrix."""
+    n = n_rows * row_elements
+    print(f"case rows kind={kind} rows={n_rows} row_elements={row_elements}", flush=True)
+    w = make_case(kind, n, 91)
+    c = compress_product(w)
+    ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"], c["output_positions"], c["gaps"])
+    assert np.array_equal(ref, w)
+    g = to_gpu(c)
+    ws, max_sub = D.prepare(g["luts"].contiguous(), g["encoded_exponent"], g["output_positions"], g["gaps"], n)
+    rng = np.random.default_rng(17)
+    for n_ids in (1, 5, 64):
+        ids = rng.integers(0, n_rows, n_ids)
+        ids[0] = n_rows - 1
+        if n_ids > 2:
+            ids[1], ids[2] = 0, ids[0]
+        asked = np.concatenate([ids, [-1, n_rows, n_rows + 5, 2 ** 40]]) if n_ids > 1 else ids
+        rng.shuffle(asked)
+        sentinel = 0xEEEE
+        out = torch.full((n,), sentinel - 65536, dtype=torch.int16, device=DEV).view(torch.bfloat16)
+        D.decode_rows(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
+                      out, ws, max_sub, torch.from_numpy(asked.astype(np.int64)).to(DEV), row_elements)
+        torch.cuda.synchronize()
+        got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+        wanted = np.zeros(n, bool)
+        for i in ids:
+            wanted[i * row_elements:(i + 1) * row_elements] = True
+        assert np.array_equal(got[wanted], w[wanted]), (kind, n_ids)
+        written = got != sentinel
+        assert np.array_equal(got[written], w[written]), (kind, n_ids)       # whatever else was written is right too
+        # a sub-block holds at most 4096 elements: nothing further than that from a requested row is touched
+        near = np.zeros(n + 1, np.int64)
+        for i in ids:
+            near[max(0, i * row_elements - 4096)] += 1
+            near[min(n, (i + 1) * row_elements + 4096)] -= 1
+        far = np.cumsum(near[:-1]) == 0
+        assert not (written & far & (w != sentinel)).any(), (kind, n_ids)
