@@ -552,7 +552,7 @@ __device__ __forceinline__ void decode_body(
   }
 }
 
-// Launch plans.  The kernel is one body compiled three ways; which one runs is
+// Launch plans.  The kernel is one body compiled for three plans; which one runs is
 // decided per stream at launch time from two numbers the host knows, the number of
 // sub-blocks and the elements an average sub-block produces.  Measured on MI355X
 // (N(0, 0.02), Laplace, one-bit and incompressible streams of 17 M to 622 M
@@ -574,7 +574,11 @@ __device__ __forceinline__ void decode_body(
 // sub-blocks per wavefront, which sets wavefront priorities by phase (see the loop),
 // and `deep` in a third (`_small`) that also reads with plain loads, for the streams
 // under 38 M elements that fit its rounds better than those of `wide` (a stream that
-// small may still sit in the memory-side cache).
+// small may still sit in the memory-side cache).  `wide` has a second compilation as
+// well (`_full`: four workgroups per CU, eight wavefronts per SIMD, priorities by
+// phase) for the streams whose sub-blocks fit one round of that many wavefronts but
+// not one round of `wide`.  `portable` is `wide` with LDS addressed through its symbol
+// (see decode_body), and `rows` serves df11_decode_rows.
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
 #define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd, const_lds)  \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
@@ -592,6 +596,7 @@ DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4, true)
 DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4, true)
 DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4, true)
 DF11_DECODE_KERNEL(decode_kernel_portable, 2, false, false, 6, false)   // `wide`, LDS addressed through its symbol
+DF11_DECODE_KERNEL(decode_kernel_wide_full, 2, false, true, 8, true)    // `wide` at four workgroups per CU
 #undef DF11_DECODE_KERNEL
 
 // Decodes only the sub-blocks that hold given rows of the output matrix (an embedding
@@ -614,6 +619,7 @@ struct LaunchPlan {
 };
 constexpr int kWideGroupsPerCu = 3;
 constexpr int kDeepGroupsPerCu = 2;
+constexpr int kFullGroupsPerCu = 4;   // 8 wavefronts per SIMD: every one the registers of `wide` allow
 constexpr int kMinElemsPerWaveForDeep = 6144;  // output per resident wavefront of the wide plan: four typical sub-blocks
 constexpr int kMinElemsPerSubForDeep = 1024;   // below: more than 4 bits per exponent, decode-bound
 constexpr int kMinElemsPerSubForDeepest = 2560;
@@ -625,6 +631,7 @@ constexpr int kMaxRoundsForPhasePriority = 16;
 constexpr int64_t kMaxInputBytesForPlainLoads = 40 << 20;   // about 30 M weight-like elements
 
 const LaunchPlan kWide{decode_kernel_wide, kWideGroupsPerCu, nullptr, "wide", nullptr};
+const LaunchPlan kWideFull{decode_kernel_wide_full, kFullGroupsPerCu, nullptr, "wide/full", nullptr};
 const LaunchPlan kDeep{decode_kernel_deep, kDeepGroupsPerCu, decode_kernel_deep_short, "deep", "deep/short"};
 const LaunchPlan kDeepSmall{decode_kernel_deep_small, kDeepGroupsPerCu, decode_kernel_deep_small, "deep/small",
                             "deep/small"};
@@ -646,17 +653,25 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned =
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
   if (elems_per_sub < kMinElemsPerSubForDeep) return kWide;
   if (n_elements < kMinElemsPerWaveForDeep * wide_waves) {
-    // A few rounds of sub-blocks.  Under the wide plan such a launch takes as long as
-    // its rounds, full or not: 0.79 W + ceil(n / W) W in units of one sub-block's share
-    // of a full round of W wavefronts.  Under the deep plan it grows evenly with the
-    // stream, 1.08 W + 0.91 n (measured from 2,500 to 24,000 sub-blocks read from HBM),
-    // within 0.25 W up to two rounds of W and proportionally closer beyond: kept as
-    // margin.  Short-code streams stay wide.
+    // A few rounds of sub-blocks.  Short-code streams stay wide.
+    if (elems_per_sub >= kMinElemsPerSubForDeepest) return kWide;
+    // The second round of the wide plan's W wavefronts.  Up to the wavefronts that four
+    // workgroups per CU have, one round of those instead of a full round and a nearly
+    // empty one (10 M elements 13.4 -> 12.0 us, 12 M 14.6 -> 12.6 us; below one round of
+    // W, and from 13 M to 17 M elements, four per CU are no faster or 4-9 % slower); the
+    // rest of the second round stays wide (13 M elements: 14.6 us against 16.9 us under
+    // the deep plan, whose own third round starts there).
+    const int64_t full_waves = (int64_t)cus * kFullGroupsPerCu * kWavesPerGroup;
+    if (n_subs > wide_waves && n_subs <= 2 * wide_waves) return n_subs <= full_waves ? kWideFull : kWide;
+    // Elsewhere: under the wide plan such a launch takes as long as its rounds, full or
+    // not: 0.79 W + ceil(n / W) W in units of one sub-block's share of a full round.  Under
+    // the deep plan it grows more evenly with the stream, 1.08 W + 0.91 n (measured from
+    // 2,500 to 24,000 sub-blocks read from HBM), within 0.25 W up to two rounds of W and
+    // proportionally closer beyond: kept as margin.
     const int64_t wide_cost = (79 * wide_waves + (n_subs + wide_waves - 1) / wide_waves * wide_waves * 100);
     const int64_t margin = n_subs > 2 * wide_waves ? 25 * wide_waves * 2 * wide_waves / n_subs : 25 * wide_waves;
     const int64_t deep_cost = 108 * wide_waves + margin + 91 * n_subs;
-    if (elems_per_sub >= kMinElemsPerSubForDeepest || (n_subs > deep_waves && wide_cost <= deep_cost))
-      return kWide;
+    if (n_subs > deep_waves && wide_cost <= deep_cost) return kWide;
     // Plain loads pay when the stream may still be in the memory-side cache and cost 1-5 %
     // when it comes from HBM, more the larger it is.
     const int64_t input_bytes = n_subs * kSubBytes + n_elements;
@@ -695,6 +710,7 @@ int device_info(DeviceInfo& info) {
                           reinterpret_cast<const void*>(decode_kernel_deep_small),
                           reinterpret_cast<const void*>(decode_kernel_deepest),
                           reinterpret_cast<const void*>(decode_kernel_deepest_short),
+                          reinterpret_cast<const void*>(decode_kernel_wide_full),
                           reinterpret_cast<const void*>(decode_kernel_rows)}) {
       hipFuncAttributes attr;
       e = hipFuncGetAttributes(&attr, k);

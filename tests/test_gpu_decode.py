@@ -441,3 +441,23 @@ def test_gpu_rows_match_full_decode(oracle, kind, n_rows, row_elements):
             near[min(n, (i + 1) * row_elements + 4096)] -= 1
         far = np.cumsum(near[:-1]) == 0
         assert not (written & far & (w != sentinel)).any(), (kind, n_ids)
+
+
+@pytest.mark.parametrize("kind", ["normal", "laplace", "outliers"])
+def test_gpu_stream_of_one_round_of_four_workgroups_per_cu(oracle, kind):
+    """Streams of 10 M to 12.9 M weight-like elements run the compilation of the wide plan
+    that keeps four workgroups per CU resident; the library says so without a GPU, and the
+    decode equals the oracle's and the original words."""
+    from dfloat11_amd import _native
+    n = 11_000_003
+    print(f"case wide/full kind={kind} n={n}", flush=True)
+    w = make_case(kind, n, 23)
+    c = compress_product(w)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    name = _native.hip_lib().df11_launch_plan_name(c["encoded_exponent"].size, n, cus).decode()
+    if cus == 256:
+        assert name == "wide/full", name
+    ref = oracle.c_decode(c["luts"], c["encoded_exponent"], c["sign_mantissa"], c["output_positions"], c["gaps"])
+    assert np.array_equal(ref, w)
+    assert np.array_equal(gpu_decode(c), ref)
+    assert np.array_equal(gpu_decode(c, max_elems=0, pad_front=4), ref)
