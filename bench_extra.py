@@ -3,7 +3,8 @@
 
   --workload mixes         decode GB/s and bit-exactness per adversarial exponent
                            distribution, on a 151936x4096 embedding-shaped tensor and
-                           a 4096x14336 matrix
+                           a 4096x14336 matrix, with the input read from HBM (device
+                           copies decoded in turn) and from the memory-side cache
   --workload sizes         N(0, 0.02) tensors of 2 M to 120 M elements: which compilation
                            of the kernel the library launches, and the time per launch
                            with the input read from HBM (device copies decoded in turn)
@@ -58,81 +59,15 @@ def make_mix(torch, kind, n, device, seed):
     raise ValueError(kind)
 
 
-def time_decode(torch, w, steps, warmup, preheat_ms=150.0):
-    """Encode w on the host, decode it `steps` times on the device; returns a result dict."""
-    from dfloat11_amd import decode as D
-    from dfloat11_amd import dfloat11_utils as U
-    dev = w.device
-    w_cpu = w.cpu().flatten()
-    t0 = time.perf_counter()
-    _, counter = U.get_codec(w_cpu)
-    codec, _, table = U.get_32bit_codec(counter)
-    luts = U.get_luts(table)
-    enc, sm, pos, gaps, _ = U.encode_weights([w_cpu], codec)
-    t_encode = time.perf_counter() - t0
-    d_luts, d_enc, d_sm, d_gaps = (t.to(dev) for t in (luts, enc, sm, gaps))
-    d_pos = pos.view(torch.uint8).to(dev)
-    n = w_cpu.numel()
-    ws, max_sub = D.prepare(d_luts, d_enc, d_pos, d_gaps, n)
-    out = torch.empty(n, dtype=torch.bfloat16, device=dev)
-    D.decode(d_luts, d_enc, d_sm, d_pos, d_gaps, out, ws, max_sub)   # once through the checked wrapper
-    # then the C-ABI entry point with its arguments bound once, as in bench.py
-    from dfloat11_amd import _native
-    lib = _native.hip_lib()
-    args = (d_luts.data_ptr(), d_enc.data_ptr(), d_sm.data_ptr(), d_pos.data_ptr(), d_gaps.data_ptr(),
-            out.data_ptr(), int(luts.shape[0]), int(enc.numel()), int(n), ws.data_ptr(), int(max_sub),
-            torch.cuda.current_stream(dev).cuda_stream)
-    # the host-side encode above leaves the device idle long enough for its clock to drop:
-    # launch for a while before the counted warm-up (compute-bound mixes feel the clock most)
-    t0 = time.perf_counter()
-    while (time.perf_counter() - t0) * 1e3 < preheat_ms:
-        for _ in range(16):
-            lib.df11_decode(*args)
-        torch.cuda.synchronize()
-    for _ in range(warmup):
-        lib.df11_decode(*args)
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    for i in range(steps):
-        starts[i].record()
-        if lib.df11_decode(*args) != 0:
-            raise RuntimeError("df11_decode failed")
-        ends[i].record()
-    torch.cuda.synchronize()
-    ms = float(np.median([s.elapsed_time(e) for s, e in zip(starts, ends)]))
-    # the same number of launches back to back, one event pair around them: what a launch
-    # costs when the next one is already queued behind it, as between the blocks of a model
-    # (an event between two launches leaves the device idle for a moment, which a kernel of
-    # a few tens of microseconds feels)
-    b0, b1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    b0.record()
-    for _ in range(steps):
-        lib.df11_decode(*args)
-    b1.record()
-    torch.cuda.synchronize()
-    ms_b2b = b0.elapsed_time(b1) / steps
-    algo = algorithmic_bytes(enc.numel(), n, luts.shape[0])
-    lengths = luts[-1].numpy()
-    return {
-        "n_elements": n, "kernel_ms_median": ms, "GBps": algo / (ms * 1e-3) / 1e9,
-        "hbm_frac": algo / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "back_to_back_ms_per_launch": ms_b2b, "back_to_back_hbm_frac": algo / (ms_b2b * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "algorithmic_bytes": algo,
-        "bit_exact": bool(torch.equal(out.view(torch.int16), w.flatten().view(torch.int16))),
-        "bits_per_exponent": 8.0 * enc.numel() / n, "max_code_bits": int(lengths.max()),
-        "distinct_exponents": int((lengths > 0).sum()), "n_luts": int(luts.shape[0]),
-        "compressed_over_bf16": (enc.numel() + n + gaps.numel() + 4 * pos.numel()) / (2.0 * n),
-        "max_elems_per_subblock": int(max_sub), "encode_seconds_host": t_encode,
-    }
-
-
 SIZES_M = (2, 4, 6, 8, 10, 12, 14, 16.777216, 20, 23, 25, 28, 30, 34, 37, 38, 45, 58.720256, 80, 100, 120)
 
 
-def time_copies_in_turn(torch, w, launches=40, preheat_ms=150.0):
+def time_copies_in_turn(torch, w, launches=40, preheat_ms=150.0, regimes=("hbm", "cache")):
     """Encode w once, keep enough device copies of the stream that a launch never finds its
     input in the 256 MB memory-side cache (at least 600 MB of inputs in all), and decode them
-    in turn, back to back, into one output; then the first copy alone, over and over."""
+    in turn, back to back, into one output ("hbm"); then the first copy alone, over and over
+    ("cache").  `regimes` names which of the two to run (under a profiler a run with one of
+    them holds timed launches of one kind only); the other's figures are None."""
     from dfloat11_amd import _native
     from dfloat11_amd import decode as D
     from dfloat11_amd import dfloat11_utils as U
@@ -180,9 +115,13 @@ def time_copies_in_turn(torch, w, launches=40, preheat_ms=150.0):
             times.append(b0.elapsed_time(b1) / launches)
         return float(np.median(times))
 
-    in_turn = per_launch(lambda i: i % n_copies)
-    same = per_launch(lambda i: 0)
+    in_turn = per_launch(lambda i: i % n_copies) if "hbm" in regimes else None
+    same = per_launch(lambda i: 0) if "cache" in regimes else None
     algo = algorithmic_bytes(enc.numel(), n, luts.shape[0])
+
+    def frac(ms):
+        return None if ms is None else algo / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS
+
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     lengths = luts[-1].numpy()
     return {
@@ -191,9 +130,9 @@ def time_copies_in_turn(torch, w, launches=40, preheat_ms=150.0):
         "compressed_over_bf16": input_bytes / (2.0 * n),
         "kernel": "decode_kernel_" + lib.df11_launch_plan_name(int(enc.numel()), int(n), cus).decode().replace("/", "_"),
         "device_copies": n_copies, "copies_in_turn_ms_per_launch": in_turn,
-        "copies_in_turn_hbm_frac": algo / (in_turn * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "same_copy_ms_per_launch": same, "same_copy_hbm_frac": algo / (same * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "bit_exact": bit_exact,
+        "copies_in_turn_hbm_frac": frac(in_turn),
+        "same_copy_ms_per_launch": same, "same_copy_hbm_frac": frac(same),
+        "max_elems_per_subblock": int(calls[0][10]), "bit_exact": bit_exact,
     }
 
 
@@ -214,7 +153,7 @@ def run_mixes(a, torch, dev):
     for kind in ([a.mix] if a.mix else MIXES):
         for name, rows, cols in ([t for t in ALL_SHAPES if t[0] == a.tensor] if a.tensor else MIX_SHAPES):
             w = make_mix(torch, kind, rows * cols, dev, seed=7)
-            r = time_decode(torch, w, a.steps, a.warmup)
+            r = time_copies_in_turn(torch, w, regimes=("hbm", "cache") if a.regime == "both" else (a.regime,))
             del w
             torch.cuda.empty_cache()
             ok = ok and r["bit_exact"]
@@ -437,8 +376,9 @@ def main():
     ap.add_argument("--workload", choices=["mixes", "sizes", "flux-offload"], required=True)
     ap.add_argument("--mix", choices=MIXES + ("normal",), default=None, help="mixes: only this distribution")
     ap.add_argument("--tensor", choices=[t[0] for t in ALL_SHAPES], default=None, help="mixes: only this tensor")
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--regime", choices=["hbm", "cache", "both"], default="both",
+                    help="mixes: decode device copies of the stream in turn (inputs from HBM), one copy over and "
+                         "over (inputs from the memory-side cache where they fit), or one after the other")
     ap.add_argument("--double_blocks", type=int, default=19)
     ap.add_argument("--single_blocks", type=int, default=38)
     ap.add_argument("--image_tokens", type=int, default=4096)

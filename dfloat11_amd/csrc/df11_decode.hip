@@ -653,25 +653,26 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned =
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
   if (elems_per_sub < kMinElemsPerSubForDeep) return kWide;
   if (n_elements < kMinElemsPerWaveForDeep * wide_waves) {
-    // A few rounds of sub-blocks.  Short-code streams stay wide.
+    // A few rounds of sub-blocks: the launch is bound by latency, and what counts is how
+    // the sub-blocks fill the rounds of the wavefronts a plan keeps resident (W = 6144 on
+    // 256 CUs for wide, 2/3 W for deep, 4/3 W for wide/full).  Under the wide plan such a
+    // launch takes as long as its rounds, full or not; under the deep plan it grows more
+    // evenly with the stream.  Measured on N(0, 0.02) streams of 2 M to 38 M elements read
+    // from HBM (time per launch, best plan against the next):
+    //   up to one round of deep               deep/small  (4 M elements: 7.8 against 8.4 us)
+    //   up to one round of wide               wide        (8 M: 9.7 against 10.4 us)
+    //   up to one round of wide/full          wide/full   (10 M: 12.0 against 13.4 us, 12 M: 12.6
+    //                                                      against 14.6 us: one round instead of
+    //                                                      a full one and a nearly empty one)
+    //   the rest of wide's second round       wide        (13 M: 14.7 against 16.9 us, 16.8 M: 17.1
+    //                                                      against 17.6 us)
+    //   beyond                                deep        (20 M: 19.3 against 20.9 us, 28 M: 23.6
+    //                                                      against 26.0 us)
+    // Short-code streams stay wide.
     if (elems_per_sub >= kMinElemsPerSubForDeepest) return kWide;
-    // The second round of the wide plan's W wavefronts.  Up to the wavefronts that four
-    // workgroups per CU have, one round of those instead of a full round and a nearly
-    // empty one (10 M elements 13.4 -> 12.0 us, 12 M 14.6 -> 12.6 us; below one round of
-    // W, and from 13 M to 17 M elements, four per CU are no faster or 4-9 % slower); the
-    // rest of the second round stays wide (13 M elements: 14.6 us against 16.9 us under
-    // the deep plan, whose own third round starts there).
     const int64_t full_waves = (int64_t)cus * kFullGroupsPerCu * kWavesPerGroup;
-    if (n_subs > wide_waves && n_subs <= 2 * wide_waves) return n_subs <= full_waves ? kWideFull : kWide;
-    // Elsewhere: under the wide plan such a launch takes as long as its rounds, full or
-    // not: 0.79 W + ceil(n / W) W in units of one sub-block's share of a full round.  Under
-    // the deep plan it grows more evenly with the stream, 1.08 W + 0.91 n (measured from
-    // 2,500 to 24,000 sub-blocks read from HBM), within 0.25 W up to two rounds of W and
-    // proportionally closer beyond: kept as margin.
-    const int64_t wide_cost = (79 * wide_waves + (n_subs + wide_waves - 1) / wide_waves * wide_waves * 100);
-    const int64_t margin = n_subs > 2 * wide_waves ? 25 * wide_waves * 2 * wide_waves / n_subs : 25 * wide_waves;
-    const int64_t deep_cost = 108 * wide_waves + margin + 91 * n_subs;
-    if (n_subs > deep_waves && wide_cost <= deep_cost) return kWide;
+    if (n_subs > deep_waves && n_subs <= 2 * wide_waves)
+      return n_subs > wide_waves && n_subs <= full_waves ? kWideFull : kWide;
     // Plain loads pay when the stream may still be in the memory-side cache and cost 1-5 %
     // when it comes from HBM, more the larger it is.
     const int64_t input_bytes = n_subs * kSubBytes + n_elements;
