@@ -591,6 +591,32 @@ DF11_HD int64_t workspace_bytes(int64_t n_blocks) {
   return (kWsSubposOffset + 4 * (n_blocks * kSubsPerBlock + 1) + 15) & ~(int64_t)15;
 }
 
+// ---- search over the sub-block positions (row decode) -----------------------------
+// Which sub-block holds output element `start`: the last entry of the ascending
+// positions that is <= start.  The 64 lanes of a wavefront probe 64 evenly spaced
+// entries of the remaining range at a time, so 2^24 entries take four dependent loads.
+// The range [lo, hi) always holds the answer and its first entry is <= start (entry 0 of
+// the positions is 0).
+struct SubSearch {
+  uint32_t lo, hi;
+};
+DF11_HD bool search_last_step(const SubSearch& r) { return r.hi - r.lo <= (uint32_t)kLanes; }
+DF11_HD uint32_t search_stride(const SubSearch& r) {
+  return search_last_step(r) ? 1u : (r.hi - r.lo + (uint32_t)kLanes - 1u) / (uint32_t)kLanes;
+}
+// Entry that `lane` probes, and whether it lies inside the range (a lane outside says no).
+DF11_HD uint32_t search_probe(const SubSearch& r, uint32_t lane) { return r.lo + lane * search_stride(r); }
+// `yes` lanes found their entry <= start: a run from lane 0, which is one of them (at
+// least one is assumed, so that positions that do not ascend cannot lead anywhere odd).
+// On the last step the answer is the range's `lo`.
+DF11_HD SubSearch search_narrow(const SubSearch& r, uint32_t yes) {
+  const uint32_t stride = search_stride(r);
+  SubSearch n;
+  n.lo = r.lo + ((yes ? yes : 1u) - 1u) * stride;
+  n.hi = n.lo + stride < r.hi ? n.lo + stride : r.hi;
+  return n;
+}
+
 // Where a sub-block lands.  The wavefront's staging area keeps the output's
 // phase modulo 8 elements (staging index i holds output element a0 + i), so
 // that 8-byte staging reads pair with 8-byte sign|mantissa loads and 16-byte

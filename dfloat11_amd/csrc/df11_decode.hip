@@ -300,25 +300,18 @@ struct RowsArgs {
 };
 
 // Index of the sub-block that holds output element `start` (< n_elements): the last
-// entry of the ascending `subpos` (n_entries of them, the first is 0) that is <= start.
-// The 64 lanes probe 64 evenly spaced entries at a time, so a search over 2^24 entries
-// takes four dependent loads.  The result is wavefront-uniform.
+// entry of the ascending `subpos` (n_entries of them, the first is 0) that is <= start
+// (SubSearch in df11_core.h).  The result is wavefront-uniform.
 __device__ __forceinline__ uint32_t find_sub(const uint32_t* __restrict__ subpos, uint32_t n_entries,
                                              uint32_t start, uint32_t lane) {
-  uint32_t lo = 0, hi = n_entries;   // the answer lies in [lo, hi) and subpos[lo] <= start
-  while (hi - lo > (uint32_t)kLanes) {
-    const uint32_t step = (hi - lo + (uint32_t)kLanes - 1u) / (uint32_t)kLanes;
-    const uint32_t probe = lo + lane * step;
-    const bool le = probe < hi && subpos[probe] <= start;
-    // ascending entries: the lanes that say yes are a run from lane 0, which is one of them
-    // (at least one is assumed, so that entries that do not ascend cannot lead anywhere odd)
-    const uint32_t k = max(1u, (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le)));
-    lo += (k - 1u) * step;
-    hi = min(hi, lo + step);
+  SubSearch r{0u, n_entries};
+  for (;;) {
+    const bool last = search_last_step(r);
+    const uint32_t probe = search_probe(r, lane);
+    const bool le = probe < r.hi && subpos[probe] <= start;
+    r = search_narrow(r, (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le)));
+    if (last) return r.lo;
   }
-  const uint32_t probe = lo + lane;
-  const bool le = probe < hi && subpos[probe] <= start;
-  return lo + max(1u, (uint32_t)__builtin_popcountll(__builtin_amdgcn_ballot_w64(le))) - 1u;
 }
 
 template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, bool kConstantLdsBase, bool kRows = false>
@@ -660,19 +653,18 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned =
     // evenly with the stream.  Measured on N(0, 0.02) streams of 2 M to 38 M elements read
     // from HBM (time per launch, best plan against the next):
     //   up to one round of deep               deep/small  (4 M elements: 7.8 against 8.4 us)
-    //   up to one round of wide               wide        (8 M: 9.7 against 10.4 us)
-    //   up to one round of wide/full          wide/full   (10 M: 12.0 against 13.4 us, 12 M: 12.6
-    //                                                      against 14.6 us: one round instead of
-    //                                                      a full one and a nearly empty one)
-    //   the rest of wide's second round       wide        (13 M: 14.7 against 16.9 us, 16.8 M: 17.1
+    //   up to one round of wide/full          wide/full   (8 M: 9.6 against 9.9 us; 10 M: 12.0 against
+    //                                                      13.4 us, 12 M: 12.6 against 14.6 us: one
+    //                                                      round instead of a full round of wide
+    //                                                      and a nearly empty one)
+    //   up to two rounds of wide              wide        (13 M: 14.7 against 16.9 us, 16.8 M: 17.1
     //                                                      against 17.6 us)
-    //   beyond                                deep        (20 M: 19.3 against 20.9 us, 28 M: 23.6
+    //   beyond                                deep        (20 M: 19.3 against 20.9 us, 28 M: 24.4
     //                                                      against 26.0 us)
     // Short-code streams stay wide.
     if (elems_per_sub >= kMinElemsPerSubForDeepest) return kWide;
     const int64_t full_waves = (int64_t)cus * kFullGroupsPerCu * kWavesPerGroup;
-    if (n_subs > deep_waves && n_subs <= 2 * wide_waves)
-      return n_subs > wide_waves && n_subs <= full_waves ? kWideFull : kWide;
+    if (n_subs > deep_waves && n_subs <= 2 * wide_waves) return n_subs <= full_waves ? kWideFull : kWide;
     // Plain loads pay when the stream may still be in the memory-side cache and cost 1-5 %
     // when it comes from HBM, more the larger it is.
     const int64_t input_bytes = n_subs * kSubBytes + n_elements;

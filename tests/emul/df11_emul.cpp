@@ -92,11 +92,15 @@ extern "C" int df11_emul_prepare(const uint8_t* luts, const uint8_t* codes, cons
 // Same data arguments as df11_decode (include/df11.h), host pointers; `grid`
 // plays gridDim.x (workgroups of eight wavefronts).  max_elems_per_sub <= 0
 // selects the worst case, as in the library.
-extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
-                                const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
-                                int n_luts, int64_t n_bytes, int64_t n_elements,
-                                int max_elems_per_sub, int grid, int codes_misalign,
-                                int out_misalign, int flags) {
+// The decode kernel's steps, for a whole stream (row_ids null: sub-blocks in the order
+// the persistent grid takes them) or for the rows `row_ids` of the output matrix only
+// (df11_decode_rows: `out` comes in holding what the caller's buffer held, and only the
+// sub-blocks that overlap the rows are decoded into it).
+static int emul_run(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
+                    const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
+                    int n_luts, int64_t n_bytes, int64_t n_elements,
+                    int max_elems_per_sub, int grid, int codes_misalign,
+                    int out_misalign, int flags, const int64_t* row_ids, int64_t n_ids, int64_t row_elements) {
   if (max_elems_per_sub <= 0 || max_elems_per_sub > kMaxElemsPerSub) max_elems_per_sub = kMaxElemsPerSub;
   const int64_t n_blocks = (n_bytes + kBlockBytes - 1) / kBlockBytes;
   const int64_t n_subs = (n_bytes + kSubBytes - 1) / kSubBytes;
@@ -117,6 +121,7 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   Exact<uint16_t> c_out((size_t)n_elements + out_misalign);
   uint16_t* out_p = c_out.p + out_misalign;
   memset(c_out.p, 0xEE, ((size_t)n_elements + out_misalign) * 2);
+  if (row_ids) memcpy(out_p, out, (size_t)n_elements * 2);
   Exact<uint8_t> ws((size_t)workspace_bytes(n_blocks));
   df11_emul_prepare(luts, codes_p, c_pos.p, c_gaps.p, n_luts, n_bytes, n_elements, ws.p);
   Exact<uint8_t> blob((size_t)tables_bytes(n_rows));   // what a workgroup copies into LDS
@@ -142,8 +147,8 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
   std::vector<ChunkSyms> regs(kLanes);
   const bool force_two_pass = (flags & 1) != 0;   // exercise the fall-back route on any input
   const bool force_check = true;
-  for (int64_t wave_gid = 0; wave_gid < stride; ++wave_gid) {
-    for (int64_t sub = wave_gid; sub < n_subs; sub += stride) {
+  auto do_sub = [&](int64_t sub) -> int {
+    {
       // one decode per chunk into "registers"; the wavefront falls back to the
       // two-pass route if any lane overflowed its slots or may not write everything
       bool all_fit = true;
@@ -194,14 +199,70 @@ extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const
       }
       memset(stage.p, 0, stage_used(p));
     }
+    return 0;
+  };
+  if (!row_ids) {
+    for (int64_t wave_gid = 0; wave_gid < stride; ++wave_gid)
+      for (int64_t sub = wave_gid; sub < n_subs; sub += stride)
+        if (int rc = do_sub(sub)) return rc;
+  } else {
+    // as decode_kernel_rows: per id, the sub-block that holds the row's first element
+    // (64 lanes probing the positions at a time), then sub-blocks until one starts past the row
+    const uint32_t n_entries = (uint32_t)(n_blocks * kSubsPerBlock + 1);
+    const int64_t n_rows_total = row_elements > 0 ? n_elements / row_elements : 0;
+    Exact<uint32_t> pos_copy((size_t)n_entries);
+    memcpy(pos_copy.p, subpos, (size_t)n_entries * 4);
+    for (int64_t i = 0; i < n_ids; ++i) {
+      const int64_t id = row_ids[i];
+      if (id < 0 || id >= n_rows_total) continue;
+      const int64_t first = id * row_elements, end = first + row_elements;
+      SubSearch r{0u, n_entries};
+      uint32_t s0;
+      for (;;) {
+        const bool last = search_last_step(r);
+        uint32_t yes = 0;
+        for (uint32_t lane = 0; lane < (uint32_t)kLanes; ++lane) {
+          const uint32_t probe = search_probe(r, lane);
+          if (probe < r.hi && pos_copy.p[probe] <= (uint32_t)first) ++yes;
+        }
+        r = search_narrow(r, yes);
+        if (last) { s0 = r.lo; break; }
+      }
+      if (!(pos_copy.p[s0] <= (uint32_t)first && (s0 + 1 >= n_entries || pos_copy.p[s0 + 1] > (uint32_t)first)))
+        return 9;   // the search must land on the sub-block that holds the element
+      for (int64_t s = s0; s < n_subs; ++s) {
+        if ((int64_t)pos_copy.p[s] >= end) break;
+        if (int rc = do_sub(s)) return rc;
+      }
+    }
   }
   memcpy(out, out_p, (size_t)n_elements * 2);
   return 0;
 }
 
+extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
+                                const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
+                                int n_luts, int64_t n_bytes, int64_t n_elements,
+                                int max_elems_per_sub, int grid, int codes_misalign,
+                                int out_misalign, int flags) {
+  return emul_run(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes, n_elements, max_elems_per_sub,
+                  grid, codes_misalign, out_misalign, flags, nullptr, 0, 0);
+}
+
+// Host counterpart of df11_decode_rows; `out` holds the caller's buffer on entry.
+extern "C" int df11_emul_decode_rows(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
+                                     const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
+                                     int n_luts, int64_t n_bytes, int64_t n_elements, int max_elems_per_sub,
+                                     const int64_t* row_ids, int64_t n_ids, int64_t row_elements) {
+  if (!row_ids || row_elements <= 0) return 1;
+  return emul_run(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes, n_elements, max_elems_per_sub,
+                  1, 0, 0, 0, row_ids, n_ids, row_elements);
+}
+
 #ifdef DF11_EMUL_MAIN
 // Stand-alone driver (built with AddressSanitizer): reads one case from a file
 //   i64 n_luts, n_bytes, n_elements, n_blocks, max_elems, grid, codes_misalign, out_misalign, flags
+//   (flags bit 2: df11_decode_rows for a fixed choice of rows instead of the whole stream)
 //   luts | codes | sign_mantissa | positions (n_blocks u32) | gaps
 // and writes the decoded u16 words to the output file.
 #include <cstdio>
@@ -223,8 +284,21 @@ int main(int argc, char** argv) {
             fread(gaps.p, 1, (size_t)n_blocks * kGapBytesPerBlock, f) == (size_t)n_blocks * kGapBytesPerBlock;
   fclose(f);
   if (!ok) return 2;
-  int rc = df11_emul_decode(luts.p, codes.p, sm.p, pos.p, gaps.p, out.p, (int)n_luts, n_bytes,
-                            n_elements, (int)h[4], (int)h[5], (int)h[6], (int)h[7], (int)h[8]);
+  int rc;
+  if (h[8] & 4) {
+    // rows mode: the output as a matrix of seven rows (the rest of the elements belong to
+    // no row), rows 6, 0, 3 and 3 again and three numbers outside it, into a buffer of 0xEEEE
+    const int64_t row_elements = n_elements / 7 > 0 ? n_elements / 7 : 1;
+    Exact<int64_t> ids(7);
+    const int64_t want[7] = {6, 0, 3, 3, -1, 7 + n_elements, 99};
+    memcpy(ids.p, want, sizeof want);
+    memset(out.p, 0xEE, (size_t)n_elements * 2);
+    rc = df11_emul_decode_rows(luts.p, codes.p, sm.p, pos.p, gaps.p, out.p, (int)n_luts, n_bytes, n_elements,
+                               (int)h[4], ids.p, 7, row_elements);
+  } else {
+    rc = df11_emul_decode(luts.p, codes.p, sm.p, pos.p, gaps.p, out.p, (int)n_luts, n_bytes,
+                          n_elements, (int)h[4], (int)h[5], (int)h[6], (int)h[7], (int)h[8]);
+  }
   if (rc) return 3;
   FILE* g = fopen(argv[2], "wb");
   if (!g) return 2;

@@ -110,8 +110,8 @@ def test_launch_plan_follows_stream_size_and_code_lengths():
     assert plan(100_000_000) == "deep/short"
     assert plan(120_000_000) == "deep"
     assert plan(4096 * 4096) == "wide"                 # 1.7 rounds of the wide plan, 2.6 of the deep one
-    assert plan(8_000_000) == "wide"
-    assert plan(10_000_000) == "wide/full"             # over one round of the wide plan, within one of four workgroups per CU
+    assert plan(8_000_000) == "wide/full"              # within one round of four workgroups per CU
+    assert plan(10_000_000) == "wide/full"             # ... also where three per CU would start a second round
     assert plan(12_500_000) == "wide/full"
     assert plan(13_500_000) == "wide"                  # the rest of the wide plan's second round
     assert plan(10_000_000, 0.125) == "wide"           # short codes stay wide

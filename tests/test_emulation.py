@@ -22,6 +22,8 @@ def emul():
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     L.df11_emul_decode.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, i32, i32, i32, i32]
     L.df11_emul_decode.restype = i32
+    L.df11_emul_decode_rows.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i64, i32, vp, i64, i64]
+    L.df11_emul_decode_rows.restype = i32
     return L
 
 
@@ -42,7 +44,9 @@ def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0, two_pa
 
 
 def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=None, two_pass=False,
-             ok_codes=(0,)):
+             ok_codes=(0,), rows=False):
+    """rows: df11_decode_rows for rows 6, 0, 3 of the output as a seven-row matrix (and numbers
+    outside it) into a buffer of 0xEEEE, instead of the whole stream."""
     n = c["sign_mantissa"].size
     n_bytes = c["encoded_exponent"].size
     n_blocks = -(-n_bytes // 4096)
@@ -50,7 +54,7 @@ def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=
     inp, outp = str(tmp_path / "case.bin"), str(tmp_path / "out.bin")
     with open(inp, "wb") as f:
         f.write(np.array([luts.shape[0], n_bytes, n, n_blocks, max_elems, grid, codes_misalign,
-                          out_misalign, 1 if two_pass else 0], np.int64).tobytes())
+                          out_misalign, (1 if two_pass else 0) | (4 if rows else 0)], np.int64).tobytes())
         f.write(luts.tobytes())
         f.write(c["encoded_exponent"].tobytes())
         f.write(c["sign_mantissa"].tobytes())
@@ -153,6 +157,13 @@ def test_emulated_kernel_under_asan(emul, tmp_path, kind, n, cm, om):
         got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
                        out_misalign=om, tmp_path=tmp_path, two_pass=two_pass)
         assert np.array_equal(got, w)
+    got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), tmp_path=tmp_path, rows=True)
+    row = max(1, n // 7)
+    for i in (6, 0, 3):
+        if (i + 1) * row <= n:
+            assert np.array_equal(got[i * row:(i + 1) * row], w[i * row:(i + 1) * row]), i
+    written = got != 0xEEEE
+    assert np.array_equal(got[written], w[written])
 
 
 def test_emulated_kernel_malformed_streams_stay_in_bounds(emul, tmp_path):
@@ -403,3 +414,43 @@ def test_emulated_kernel_long_codes_many_seeds(emul, seed):
     w = make_case("outliers", 4097 + 37 * seed, seed)
     c = compress_product(w)
     assert np.array_equal(run_emul(emul, c, max_elems=max_elems_per_block(c["output_positions"]), grid=2), w)
+
+
+@pytest.mark.parametrize("kind,n_rows,row_elements", [("normal", 700, 512), ("zeros", 900, 256), ("uniform256", 300, 320),
+                                                     ("fib", 2000, 64), ("laplace", 5, 30_011), ("outliers", 40_000, 3),
+                                                     ("single", 1, 1)])
+def test_emulated_row_decode(emul, kind, n_rows, row_elements):
+    """The steps of df11_decode_rows on the host: the search for the sub-block that holds a
+    row's first element lands on it (the emulation checks that), the requested rows come
+    out as the original words, whatever else is written is right as well, and elements far
+    from every requested row keep what the buffer held."""
+    n = n_rows * row_elements
+    w = make_case(kind, n, 77)
+    c = compress_product(w)
+    luts = np.ascontiguousarray(c["luts"])
+    rng = np.random.default_rng(3)
+    for n_ids in (1, 4, 40):
+        ids = rng.integers(0, n_rows, n_ids)
+        ids[0] = n_rows - 1
+        if n_ids > 2:
+            ids[1], ids[2] = 0, ids[0]
+        asked = np.concatenate([ids, [-1, n_rows, 2 ** 40]]).astype(np.int64)
+        rng.shuffle(asked)
+        sentinel = 0xEEEE
+        out = np.full(n, sentinel, np.uint16)
+        rc = emul.df11_emul_decode_rows(_p(luts), _p(c["encoded_exponent"]), _p(c["sign_mantissa"]),
+                                        _p(c["output_positions"]), _p(c["gaps"]), _p(out), luts.shape[0],
+                                        c["encoded_exponent"].size, n, 0, _p(asked), asked.size, row_elements)
+        assert rc == 0, (kind, n_ids, rc)
+        wanted = np.zeros(n, bool)
+        for i in ids:
+            wanted[i * row_elements:(i + 1) * row_elements] = True
+        assert np.array_equal(out[wanted], w[wanted]), (kind, n_ids)
+        written = out != sentinel
+        assert np.array_equal(out[written], w[written]), (kind, n_ids)
+        near = np.zeros(n + 1, np.int64)
+        for i in ids:
+            near[max(0, i * row_elements - 4096)] += 1
+            near[min(n, (i + 1) * row_elements + 4096)] -= 1
+        far = np.cumsum(near[:-1]) == 0
+        assert not (written & far & (w != sentinel)).any(), (kind, n_ids)
