@@ -122,6 +122,6 @@ def test_launch_plan_follows_stream_size_and_code_lengths():
     assert plan(4096 * 14336, 0.125) == "deepest/short"
     assert plan(4096 * 4096, 0.125) == "wide"
     for n in (1000, 4096 * 4096, 4096 * 14336, 622_329_856):
-        assert plan(n, 1.16) == "wide"                 # decode-bound whatever the size
+        assert plan(n, 1.16) == "wide/dense"           # decode-bound whatever the size
     assert plan(4096 * 14336, cus=64) == "deep"        # the same matrix is 36 rounds on a quarter of the CUs
     assert hip.df11_launch_plan_name(0, 10, 256) == b"" and hip.df11_launch_plan_name(10, 10, 0) == b""
