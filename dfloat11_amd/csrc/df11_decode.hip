@@ -21,8 +21,9 @@
 //      bytes -> one 16-byte BF16 store per lane, contiguous across the wavefront,
 //      in batches of 64 lanes that start on 256-byte lines of the output.
 // The kernel is bound by HBM; the decode (vector instructions for a little over
-// half of the memory time on weight-like streams) is hidden under it with two or
-// three workgroups per CU (the launch plans further down).
+// half of the memory time on weight-like streams) is hidden under it with two to
+// four workgroups per CU (the launch plans further down).  df11_decode_rows runs
+// the same steps on the sub-blocks that hold given rows of the output only.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -570,8 +571,9 @@ __device__ __forceinline__ void decode_body(
 // small may still sit in the memory-side cache).  `wide` has two more compilations at
 // four workgroups per CU (eight wavefronts per SIMD, all that its registers allow):
 // `_full`, priorities by phase, for the streams whose sub-blocks fit one round of that
-// many wavefronts, and `_dense`, priorities by rotation, for decode-bound streams.  `portable` is `wide` with LDS addressed through its symbol
-// (see decode_body), and `rows` serves df11_decode_rows.
+// many wavefronts, and `_dense`, priorities by rotation, for decode-bound streams.
+// `portable` is `wide` with LDS addressed through its symbol (see decode_body), and
+// `rows` serves df11_decode_rows.
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
 #define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd, const_lds)  \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
