@@ -116,7 +116,9 @@ def side_measurements(torch, dev, embedding_shape=True):
     mixes, sizes = {}, {}
     shapes = [(4096, 14336)] + ([(151936, 4096)] if embedding_shape else [])
     for rows, cols in shapes:
-        for kind in ("laplace", "outliers", "uniform256", "zeros"):
+        # the four distributions of the benchmark configuration, and on the matrix two more
+        # whose chunks take many table lookups (sparse weights, six- and seven-bit codes)
+        for kind in bench_extra.MIXES + (bench_extra.EXTRA_MIXES if (rows, cols) == (4096, 14336) else ()):
             w = bench_extra.make_mix(torch, kind, rows * cols, dev, seed=7)
             mixes[f"{kind} {rows}x{cols}"] = figures(w)
             del w

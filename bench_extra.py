@@ -32,6 +32,8 @@ from bench import HBM_PEAK_GBPS, algorithmic_bytes   # noqa: E402
 MIX_SHAPES = [("embedding", 151936, 4096), ("mlp_down", 4096, 14336)]
 ALL_SHAPES = MIX_SHAPES + [("attn_proj", 4096, 4096)]
 MIXES = ("laplace", "outliers", "uniform256", "zeros")
+# two more, outside the four that the benchmark configuration names: streams whose chunks need many table lookups
+EXTRA_MIXES = ("sparse70", "alphabet100")
 
 
 def make_mix(torch, kind, n, device, seed):
@@ -56,6 +58,14 @@ def make_mix(torch, kind, n, device, seed):
         pick = torch.rand(n, generator=g, device=device) < 1e-3
         mant = torch.randint(1, 128, (n,), generator=g, device=device, dtype=torch.int16)
         return torch.where(pick, mant, bits).view(torch.bfloat16)
+    if kind == "sparse70":                     # pruned weights: 70 % exact zeros among N(0, 0.02)
+        x = (torch.randn(n, generator=g, device=device) * 0.02).to(torch.bfloat16)
+        keep = torch.rand(n, generator=g, device=device) >= 0.7
+        return torch.where(keep, x, torch.zeros_like(x))
+    if kind == "alphabet100":                  # 100 equally likely exponents: six- and seven-bit codes
+        bits = torch.randint(-32768, 32768, (n,), generator=g, device=device, dtype=torch.int32)
+        e = 20 + ((bits >> 7) & 0xFF) % 100
+        return ((bits & ~(0xFF << 7)) | (e << 7)).to(torch.int16).view(torch.bfloat16)
     raise ValueError(kind)
 
 
@@ -374,7 +384,7 @@ def run_flux(a, torch, dev):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--workload", choices=["mixes", "sizes", "flux-offload"], required=True)
-    ap.add_argument("--mix", choices=MIXES + ("normal",), default=None, help="mixes: only this distribution")
+    ap.add_argument("--mix", choices=MIXES + EXTRA_MIXES + ("normal",), default=None, help="mixes: only this distribution")
     ap.add_argument("--tensor", choices=[t[0] for t in ALL_SHAPES], default=None, help="mixes: only this tensor")
     ap.add_argument("--regime", choices=["hbm", "cache", "both"], default="both",
                     help="mixes: decode device copies of the stream in turn (inputs from HBM), one copy over and "

@@ -290,13 +290,6 @@ struct Tables {
   ConstLdsBytes cntt;    // u8[2048]
 };
 
-// Unaligned 32-/16-bit stores (LDS supports them on gfx950; one instruction each).
-DF11_HD void store32(LdsBytes p, uint32_t v) { __builtin_memcpy(p, &v, 4); }
-DF11_HD void store16(LdsBytes p, uint32_t v) {
-  const uint16_t h = (uint16_t)v;
-  __builtin_memcpy(p, &h, 2);
-}
-
 // Keeps a rarely taken branch a branch: without it the compiler turns the body
 // into unconditional selects that every loop iteration pays for.
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -342,91 +335,62 @@ DF11_HD uint32_t count_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32
   return n;
 }
 
-// Decode the first `remaining` codes of the chunk and write their symbols
-// (exponent bytes) to p[0..remaining).  While four or more bytes remain the
-// four symbol bytes of a lookup are stored at once: bytes past the codes it
-// resolved are overwritten by the next store.  The last one to three symbols
-// are gathered in a register and stored exactly, so nothing is ever written at
-// or beyond p + remaining.
+// Decode the first `remaining` codes of the chunk and OR their symbols (exponent
+// bytes) into stage[at .. at + remaining), which must hold zeros (`stage` is 4-byte
+// aligned, at >= 4).  Each lookup's symbol bytes go out as two aligned words, as in
+// replay_chunk; the last lookup is cut to the codes that remain, so nothing is
+// written at or beyond at + remaining except zeros.
 DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo, uint32_t next,
-                        uint32_t gap, uint32_t remaining, LdsBytes p) {
-  uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
-  uint32_t c = gap;                     // bit 7 is set once the look-ahead has been appended
-  uint32_t rem = remaining;
-  while (rem >= 4u) {
-    if (c - 32u < 96u) {                // 32 <= c < 128: room for the look-ahead, not yet appended
-      w |= (uint64_t)next << (c - 32u);
-      c += 128u;
-      DF11_KEEP_BRANCH();
-    }
-    const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
-    uint32_t syms = e.x, meta = e.y;
-    if (meta & kUnsettled) {
-      const uint32_t long_code = walk_from(l, syms, meta, (uint32_t)(w >> 32));   // at least 32 valid bits: c < 32, or already appended
-      syms = entry_symbol(long_code);
-      meta = entry_meta(long_code);
-      DF11_KEEP_BRANCH();
-    }
-    store32(p, syms);
-    const uint32_t k = meta >> 8;
-    p += k;
-    rem -= k;
-    w <<= (meta & 63u);
-    c += meta & 0xffu;
-  }
-  if (rem) {
-    uint32_t acc = 0, got = 0;          // got: bits gathered, 8 per symbol
-    while (got < 8u * rem) {
-      if (c - 32u < 96u) {
-        w |= (uint64_t)next << (c - 32u);
-        c += 128u;
-      }
-      const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
-      uint32_t syms = e.x, meta = e.y;
-      if (meta & kUnsettled) {
-        const uint32_t long_code = walk_from(l, syms, meta, (uint32_t)(w >> 32));
-        syms = entry_symbol(long_code);
-        meta = entry_meta(long_code);
-      }
-      acc |= syms << got;
-      got += 8u * (meta >> 8);
-      w <<= (meta & 63u);
-      c += meta & 0xffu;
-    }
-    if (rem & 2u) store16(p, acc);
-    if (rem & 1u) p[rem & 2u] = (uint8_t)(acc >> (8u * (rem & 2u)));
-  }
-}
+                        uint32_t gap, uint32_t remaining, LdsBytes stage, uint32_t at);
 
 // ---- one decode per chunk, kept in registers -------------------------------------
 // The fast path decodes a chunk once.  The lookups of a chunk are few (each
-// resolves up to four codes), so their results fit in registers: kMainSlots
-// lookups that stay inside the chunk plus kTailSlots for the codes that reach
-// into the look-ahead (a tail lookup may hold symbols of the next chunk as well:
-// they are the true next symbols of the stream).  Once the lane's output offset
-// is known, the symbols are replayed into the staging area with no further
-// table access.  A chunk that
-// needs more lookups than there are slots reports `overflow` and is handled by
-// count_chunk / emit_chunk instead.
-constexpr int kMainSlots = 7;
+// resolves up to four codes), so their results fit in registers: kMain lookups
+// that stay inside the chunk plus kTailSlots for the codes that reach into the
+// look-ahead (a tail lookup may hold symbols of the next chunk as well: they are
+// the true next symbols of the stream).  Once the lane's output offset is known,
+// the symbols are replayed into the staging area with no further table access.
+// A chunk that needs more lookups than there are slots reports `overflow` and the bit
+// at which the rest of it starts: that rest is counted by count_chunk and, once the
+// lane's offset is known, decoded a second time by emit_chunk, so the cost of running
+// out of slots grows with the lookups that did not fit.
+// How many lookups a chunk needs depends on the code: weight-like streams (2.6 bits
+// per code, 3.3 codes per lookup) need seven inside the chunk; codes of six to eight
+// bits resolve one per lookup and need up to ten; streams of one- to three-bit
+// codes (sparse weights) resolve four per lookup and need up to fourteen (a lookup
+// inside the chunk starts at bit 53 or before and consumes at least four bits
+// unless a code that does not fit the window follows).  The kernel is compiled for
+// several slot counts; slots that no lane of a wavefront uses cost a compare and a
+// branch each.  Seven is what fits the 64 registers of eight wavefronts per SIMD.
+constexpr int kMainSlotsUsual = 10;        // wide (six wavefronts per SIMD), portable, rows
+constexpr int kMainSlotsFew = 7;           // the compilations for eight wavefronts per SIMD
+constexpr int kMainSlotsDeep = 8;          // large weight-like streams: a ninth changes nothing there, a tenth costs 1 %
+constexpr int kMainSlotsShortCodes = 14;   // deepest
 constexpr int kTailSlots = 2;
-constexpr int kSlots = kMainSlots + kTailSlots;
 
+template <int kMain>
 struct ChunkSyms {
-  uint32_t syms[kSlots];   // symbol bytes of lookup i, first code in byte 0, unused bytes zero
-  uint32_t ends[kSlots - 1];   // symbols of the chunk up to and including lookup i
-  uint32_t count;          // codes that start in the chunk
-  bool overflow;           // ran out of slots: count and syms are incomplete
+  static constexpr int kSlots = kMain + kTailSlots;
+  uint32_t syms[kSlots];             // symbol bytes of lookup i, first code in byte 0, unused bytes zero
+  uint32_t ends[kSlots - 1];         // symbols of the chunk up to and including lookup i
+  uint32_t count;                    // codes that start in the chunk; if `overflow`, those of the main lookups only
+  uint32_t resume;                   // bit of the chunk at which the lookups after the main ones start
+  bool overflow;                     // ran out of slots: the codes from bit `resume` on are not in syms (the
+                                     // tail slots are empty then) and not in count
 };
 
-DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
-                                    uint32_t next, uint32_t gap) {
-  ChunkSyms r;
+// kResume: the caller continues an overflowing chunk from `resume`; without it the caller
+// decodes such a chunk again from its start and needs nothing but the flag.
+template <int kMain, bool kResume>
+DF11_HD ChunkSyms<kMain> decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo,
+                                           uint32_t next, uint32_t gap) {
+  constexpr int kSlots = ChunkSyms<kMain>::kSlots;
+  ChunkSyms<kMain> r;
   uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
   const uint64_t next31 = look_ahead(next);
   uint32_t c = gap, n = 0;
 #pragma unroll
-  for (int i = 0; i < kMainSlots; ++i) {
+  for (int i = 0; i < kMain; ++i) {
     r.syms[i] = 0;
     if (c <= 64u - (uint32_t)kK) {          // the lookup stays inside the chunk
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
@@ -445,6 +409,8 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
     r.ends[i] = n;                            // also for a lane that skipped the lookup: later ones start here
   }
   r.overflow = c <= 64u - (uint32_t)kK;
+  r.resume = c;
+  const uint32_t n_main = n;
   uint32_t todo = 0;                          // codes that still start before the chunk ends
   if (!r.overflow && c < 64u) {
     todo = t.cntt[(1u << (64u - c)) | (uint32_t)(w >> c)];
@@ -452,7 +418,7 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
   }
 #pragma unroll
   for (int i = 0; i < kTailSlots; ++i) {
-    r.syms[kMainSlots + i] = 0;
+    r.syms[kMain + i] = 0;
     if (todo) {
       const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
       uint32_t syms = e.x, meta = e.y;
@@ -461,16 +427,23 @@ DF11_HD ChunkSyms decode_chunk_regs(const Tables& t, const Rows& l, uint32_t hi,
         syms = entry_symbol(long_code);
         meta = entry_meta(long_code);
       }
-      r.syms[kMainSlots + i] = syms;
+      r.syms[kMain + i] = syms;
       const uint32_t k = meta >> 8;
       const uint32_t take = k < todo ? k : todo;
       n += take;
       todo -= take;
       w <<= (meta & 63u);
     }
-    if (kMainSlots + i < kSlots - 1) r.ends[kMainSlots + i] = n;
+    if (kMain + i < kSlots - 1) r.ends[kMain + i] = n;
   }
-  r.overflow = r.overflow || todo != 0u;
+  if (todo != 0u) {                           // more tail lookups than slots: leave the whole tail to the caller
+    r.overflow = true;
+    if (kResume) {
+#pragma unroll
+      for (int i = 0; i < kTailSlots; ++i) r.syms[kMain + i] = 0;
+      n = n_main;
+    }
+  }
   r.count = n;
   return r;
 }
@@ -498,6 +471,22 @@ DF11_HD uint32_t align_bytes(uint32_t hi, uint32_t lo, uint32_t bytes) {
 #endif
 }
 
+// Is `pred` true in any lane of the wavefront?  (On the host every lane is emulated on
+// its own and answers for itself.)
+DF11_HD bool any_lane(bool pred) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_ballot_w64(pred) != 0;
+#else
+  return pred;
+#endif
+}
+
+// Main slots from this one on are there for the streams that need them: they are skipped
+// when no lane of the wavefront holds symbols in them (symbol bytes that are all zero
+// change nothing when ORed).  The slots before it, and the tail slots, are in use in
+// nearly every wavefront of any stream.
+constexpr int kFirstOptionalSlot = 7;
+
 // OR the chunk's symbols into stage[at .. at + r.count), which must hold zeros
 // (`stage` is 4-byte aligned, at >= 4).  Each lookup's four symbol bytes go out as
 // two aligned words, shifted to their byte position; the unused bytes of a lookup
@@ -507,15 +496,55 @@ DF11_HD uint32_t align_bytes(uint32_t hi, uint32_t lo, uint32_t bytes) {
 // (-pos) & 3 bytes to the right of {symbols, 0}, which one instruction per word
 // does from -pos itself; a lookup that starts on a word boundary ORs zero into the
 // word before it.
-DF11_HD void replay_chunk(const ChunkSyms& r, LdsBytes stage, uint32_t at) {
+template <int kMain>
+DF11_HD void replay_chunk(const ChunkSyms<kMain>& r, LdsBytes stage, uint32_t at) {
   const uint32_t minus_at = 0u - at;
 #pragma unroll
-  for (int i = 0; i < kSlots; ++i) {
+  for (int i = 0; i < ChunkSyms<kMain>::kSlots; ++i) {
+    if (i >= kFirstOptionalSlot && i < kMain && !any_lane(r.syms[i] != 0u)) continue;
     // lookup i starts where the lookups before it end
     const uint32_t minus_pos = i == 0 ? minus_at : minus_at - r.ends[i - 1];
     LdsBytes w = stage + (~minus_pos & ~3u);               // (pos - 1) & ~3
     or32_aligned(w, align_bytes(r.syms[i], 0u, minus_pos));
     or32_aligned(w + 4, align_bytes(0u, r.syms[i], minus_pos));
+  }
+}
+
+DF11_HD void emit_chunk(const Tables& t, const Rows& l, uint32_t hi, uint32_t lo, uint32_t next,
+                        uint32_t gap, uint32_t remaining, LdsBytes stage, uint32_t at) {
+  uint64_t w = (((uint64_t)hi << 32) | lo) << gap;
+  uint32_t c = gap;                     // bit 7 is set once the look-ahead has been appended
+  uint32_t rem = remaining;
+  uint32_t minus_pos = 0u - at;
+  while (rem) {
+    if (c - 32u < 96u) {                // 32 <= c < 128: room for the look-ahead, not yet appended
+      w |= (uint64_t)next << (c - 32u);
+      c += 128u;
+      DF11_KEEP_BRANCH();
+    }
+    const U32x2 e = lds_load<U32x2>(t.dec + dec_offset(w));
+    uint32_t syms = e.x, meta = e.y;
+    if (meta & kUnsettled) {
+      const uint32_t long_code = walk_from(l, syms, meta, (uint32_t)(w >> 32));   // at least 32 valid bits: c < 32, or already appended
+      syms = entry_symbol(long_code);
+      meta = entry_meta(long_code);
+      DF11_KEEP_BRANCH();
+    }
+    uint32_t k = (meta >> 8) & 0xffu;
+    if (k > rem) {                      // the last lookup holds codes past the quota (k <= 4, so rem < 4)
+      syms &= (1u << (8u * rem)) - 1u;
+      k = rem;
+    }
+    LdsBytes word = stage + (~minus_pos & ~3u);            // (pos - 1) & ~3
+    if (minus_pos & 3u) {               // a lookup that starts on a word boundary has nothing for the word before it
+      or32_aligned(word, align_bytes(syms, 0u, minus_pos));
+      DF11_KEEP_BRANCH();
+    }
+    or32_aligned(word + 4, align_bytes(0u, syms, minus_pos));
+    minus_pos -= k;
+    rem -= k;
+    w <<= (meta & 63u);
+    c += meta & 0xffu;
   }
 }
 

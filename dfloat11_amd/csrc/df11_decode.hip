@@ -315,7 +315,8 @@ __device__ __forceinline__ uint32_t find_sub(const uint32_t* __restrict__ subpos
   }
 }
 
-template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, bool kConstantLdsBase, bool kRows = false>
+template <int kPrefetchGroups, bool kStreaming, bool kPhasePriority, bool kConstantLdsBase, int kMain, bool kResume,
+          bool kRows = false>
 __device__ __forceinline__ void decode_body(
     const uint8_t* __restrict__ codes,
     const uint8_t* __restrict__ sign_mantissa, const uint8_t* __restrict__ gaps,
@@ -432,12 +433,23 @@ __device__ __forceinline__ void decode_body(
     const Chunk c{__builtin_bswap32(cur.d0), __builtin_bswap32(cur.d1), __builtin_bswap32(cur.d2)};
     const uint32_t gap_word = __builtin_bswap32(cur.gap_raw) >> 16;   // the two bytes, big-endian
     const uint32_t gap = (gap_word >> gap_shift) & 31u;
-    // One decode per chunk, results held in registers.  If any lane of the
-    // wavefront ran out of register slots, or may not write all its symbols (end
-    // of the tensor), the wavefront takes the two-pass route instead.
-    const ChunkSyms cs = decode_chunk_regs(t, l, c.hi, c.lo, c.next, gap);
-    const bool all_fit = wave_all(!cs.overflow);
-    const uint32_t count = all_fit ? cs.count : count_chunk(t, l, c.hi, c.lo, c.next, gap);
+    // One decode per chunk, results held in registers.  A lane that ran out of
+    // register slots counts the rest of its chunk now and decodes that rest a second
+    // time once its offset is known.  If some lane may not write all its symbols (end
+    // of the tensor, staging smaller than the sub-block), the wavefront decodes
+    // everything a second time instead, up to each lane's quota.
+    const ChunkSyms<kMain> cs = decode_chunk_regs<kMain, kResume>(t, l, c.hi, c.lo, c.next, gap);
+    // (The compilations for eight wavefronts per SIMD have no register left for the place
+    // where a lane's rest starts: there a wavefront with such a lane counts and decodes
+    // whole chunks again.)
+    const bool redo_all = !kResume && !wave_all(!cs.overflow);
+    uint32_t count = cs.count;
+    if (redo_all) {
+      count = count_chunk(t, l, c.hi, c.lo, c.next, gap);
+    } else if (kResume && cs.overflow) {
+      count += count_chunk(t, l, c.hi, c.lo, c.next, cs.resume);
+      DF11_KEEP_BRANCH();
+    }
     const uint32_t incl = wave_inclusive_scan(count);
     const uint32_t total = wave_total(incl);                  // uniform
     const uint32_t excl = incl - count;
@@ -445,10 +457,15 @@ __device__ __forceinline__ void decode_body(
     // ---- symbols to their place in the staging area, in output order
     const SubPlan p = plan_sub((int64_t)base, total, z.n_elements, z.stage_cap);   // uniform
     const uint32_t quota = thread_quota(excl, count, p.n_out);
-    if (all_fit && wave_all(quota == count))
+    if (!redo_all && wave_all(quota == count)) {
       replay_chunk(cs, lds, stage_offset + p.phase + excl);   // one base for all: the wavefront's offset rides in the index
-    else
-      emit_chunk(t, l, c.hi, c.lo, c.next, gap, quota, stage + p.phase + excl);
+      if (kResume && cs.overflow) {
+        emit_chunk(t, l, c.hi, c.lo, c.next, cs.resume, count - cs.count, lds, stage_offset + p.phase + excl + cs.count);
+        DF11_KEEP_BRANCH();
+      }
+    } else {
+      emit_chunk(t, l, c.hi, c.lo, c.next, gap, quota, lds, stage_offset + p.phase + excl);
+    }
     // Staging is exchanged between the lanes of one wavefront only; its LDS
     // operations execute in order, the fence keeps the compiler from reordering.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -575,24 +592,24 @@ __device__ __forceinline__ void decode_body(
 // `portable` is `wide` with LDS addressed through its symbol (see decode_body), and
 // `rows` serves df11_decode_rows.
 // The register budget follows the resident wavefronts (amdgpu_waves_per_eu).
-#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd, const_lds)  \
+#define DF11_DECODE_KERNEL(name, prefetch, streaming, phase_priority, waves_per_simd, const_lds, slots) \
   __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_per_simd,       \
                                                                              waves_per_simd)))    \
   void name(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,         \
             const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,                         \
             const uint8_t* __restrict__ ws, const DecodeSizes z) {                                \
-    decode_body<prefetch, streaming, phase_priority, const_lds>(codes, sign_mantissa, gaps, out,  \
-                                                                ws, z);                           \
+    decode_body<prefetch, streaming, phase_priority, const_lds, slots, (waves_per_simd < 8)>(     \
+        codes, sign_mantissa, gaps, out, ws, z);                                                  \
   }
-DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6, true)
-DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4, true)
-DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4, true)
-DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4, true)
-DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4, true)
-DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4, true)
-DF11_DECODE_KERNEL(decode_kernel_portable, 2, false, false, 6, false)   // `wide`, LDS addressed through its symbol
-DF11_DECODE_KERNEL(decode_kernel_wide_full, 2, false, true, 8, true)    // `wide` at four workgroups per CU
-DF11_DECODE_KERNEL(decode_kernel_wide_dense, 2, false, false, 8, true)  // the same with priorities by rotation
+DF11_DECODE_KERNEL(decode_kernel_wide, 2, false, false, 6, true, kMainSlotsUsual)
+DF11_DECODE_KERNEL(decode_kernel_deep, 3, true, false, 4, true, kMainSlotsDeep)
+DF11_DECODE_KERNEL(decode_kernel_deep_short, 3, true, true, 4, true, kMainSlotsDeep)
+DF11_DECODE_KERNEL(decode_kernel_deep_small, 3, false, true, 4, true, kMainSlotsDeep)
+DF11_DECODE_KERNEL(decode_kernel_deepest, 6, true, false, 4, true, kMainSlotsShortCodes)
+DF11_DECODE_KERNEL(decode_kernel_deepest_short, 6, true, true, 4, true, kMainSlotsShortCodes)
+DF11_DECODE_KERNEL(decode_kernel_portable, 2, false, false, 6, false, kMainSlotsUsual)   // `wide`, LDS addressed through its symbol
+DF11_DECODE_KERNEL(decode_kernel_wide_full, 2, false, true, 8, true, kMainSlotsFew)    // `wide` at four workgroups per CU
+DF11_DECODE_KERNEL(decode_kernel_wide_dense, 2, false, false, 8, true, kMainSlotsFew)  // the same with priorities by rotation
 #undef DF11_DECODE_KERNEL
 
 // Decodes only the sub-blocks that hold given rows of the output matrix (an embedding
@@ -602,7 +619,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6))
 void decode_kernel_rows(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,
                         const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,
                         const uint8_t* __restrict__ ws, const DecodeSizes z, const RowsArgs rows) {
-  decode_body<2, false, true, true, true>(codes, sign_mantissa, gaps, out, ws, z, rows);
+  decode_body<2, false, true, true, kMainSlotsUsual, true, true>(codes, sign_mantissa, gaps, out, ws, z, rows);
 }
 
 typedef void (*DecodeKernel)(const uint8_t*, const uint8_t*, const uint8_t*, uint16_t*, const uint8_t*, DecodeSizes);
@@ -618,7 +635,8 @@ constexpr int kDeepGroupsPerCu = 2;
 constexpr int kFullGroupsPerCu = 4;   // 8 wavefronts per SIMD: every one the registers of `wide` allow
 constexpr int kMinElemsPerWaveForDeep = 6144;  // output per resident wavefront of the wide plan: four typical sub-blocks
 constexpr int kMinElemsPerSubForDeep = 1024;   // below: more than 4 bits per exponent, decode-bound
-constexpr int kMinElemsPerSubForDeepest = 2560;
+constexpr int kMinElemsPerSubForManyLookups = 480;   // below: codes so long that seven lookups cover a chunk
+constexpr int kMinElemsPerSubForDeepest = 2048;   // two bits per code and fewer: sparse weights, one-bit streams
 // Up to this many sub-blocks per wavefront, the deep plans set wavefront priorities by
 // phase (4096x14336 to 100 M elements: 2-7 % faster than by turn; equal at 120 M to
 // 142 M; 0.5 % slower at 218 M, 5 % at 622 M; 9 % slower under the wide plan on a
@@ -648,9 +666,13 @@ LaunchPlan plan_launch(int64_t n_subs, int64_t n_elements, int cus, int pinned =
   const int64_t wide_waves = (int64_t)cus * kWideGroupsPerCu * kWavesPerGroup;
   const int64_t deep_waves = (int64_t)cus * kDeepGroupsPerCu * kWavesPerGroup;
   const int64_t elems_per_sub = n_subs ? n_elements / n_subs : 0;
-  // Decode-bound streams gain from every wavefront the registers allow (incompressible
-  // exponents, 8 M to 622 M elements: 2.5-5 % faster at four workgroups per CU than at three).
-  if (elems_per_sub < kMinElemsPerSubForDeep) return kWideDense;
+  // Decode-bound streams.  With more than 8.5 bits per code on average (fewer than 480
+  // elements per sub-block) seven lookups cover a chunk, and the stream gains from every
+  // wavefront the registers allow (incompressible exponents, 8 M to 622 M elements: 2.5-5 %
+  // faster at four workgroups per CU than at three).  Codes of 5.5 to 8.5 bits take eight to
+  // ten lookups per chunk, which only the compilations with more register slots hold.
+  if (elems_per_sub < kMinElemsPerSubForManyLookups) return kWideDense;
+  if (elems_per_sub < kMinElemsPerSubForDeep) return kWide;
   if (n_elements < kMinElemsPerWaveForDeep * wide_waves) {
     // A few rounds of sub-blocks: the launch is bound by latency, and what counts is how
     // the sub-blocks fill the rounds of the wavefronts a plan keeps resident (W = 6144 on

@@ -6,7 +6,7 @@ import torch
 
 from dfloat11_amd import dfloat11_utils as U
 
-KINDS = ("normal", "laplace", "outliers", "uniform256", "zeros", "fib", "single", "high")
+KINDS = ("normal", "laplace", "outliers", "uniform256", "zeros", "fib", "single", "high", "sparse", "alphabet100")
 
 
 def _bf16(x):
@@ -48,6 +48,14 @@ def make_case(kind, n, seed):
         return (((sm & 0x80) << 8) | (np.uint16(121) << 7) | (sm & 0x7F)).astype(np.uint16)
     if kind == "high":            # only exponents >= 240 (huge values, Inf, NaN)
         e = rng.integers(240, 256, n).astype(np.uint16)
+        sm = rng.integers(0, 256, n).astype(np.uint16)
+        return (((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)).astype(np.uint16)
+    if kind == "sparse":          # pruned weights: 70 % exact zeros among N(0, 0.02): one-bit codes next to
+        x = rng.standard_normal(n) * 0.02                     # four- to ten-bit ones, 30 and more per chunk
+        x[rng.random(n) < 0.7] = 0.0
+        return _bf16(x)
+    if kind == "alphabet100":     # 100 equally likely exponents: six- and seven-bit codes, one per table
+        e = rng.integers(20, 120, n).astype(np.uint16)        # lookup, nine to eleven lookups per chunk
         sm = rng.integers(0, 256, n).astype(np.uint16)
         return (((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)).astype(np.uint16)
     raise ValueError(kind)

@@ -96,6 +96,7 @@ extern "C" int df11_emul_prepare(const uint8_t* luts, const uint8_t* codes, cons
 // the persistent grid takes them) or for the rows `row_ids` of the output matrix only
 // (df11_decode_rows: `out` comes in holding what the caller's buffer held, and only the
 // sub-blocks that overlap the rows are decoded into it).
+template <int kMain>
 static int emul_run(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
                     const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
                     int n_luts, int64_t n_bytes, int64_t n_elements,
@@ -144,32 +145,30 @@ static int emul_run(const uint8_t* luts, const uint8_t* codes, const uint8_t* si
 
   std::vector<Chunk> chunk(kLanes);
   std::vector<uint32_t> gap(kLanes), count(kLanes), excl(kLanes);
-  std::vector<ChunkSyms> regs(kLanes);
+  std::vector<ChunkSyms<kMain>> regs(kLanes);
   const bool force_two_pass = (flags & 1) != 0;   // exercise the fall-back route on any input
-  const bool force_check = true;
   auto do_sub = [&](int64_t sub) -> int {
     {
-      // one decode per chunk into "registers"; the wavefront falls back to the
-      // two-pass route if any lane overflowed its slots or may not write everything
-      bool all_fit = true;
+      // one decode per chunk into "registers"; a lane that ran out of slots counts the
+      // rest of its chunk, and decodes that rest again once its offset is known
       for (int lane = 0; lane < kLanes; ++lane) {
         const int64_t gid = sub * kLanes + lane;
         chunk[lane] = fetch_chunk(codes_p, n_bytes, gid, codes_aligned);
         gap[lane] = gap_of(c_gaps.p, gid, n_gap_bytes);
-        regs[lane] = decode_chunk_regs(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
-        all_fit = all_fit && !regs[lane].overflow;
+        regs[lane] = decode_chunk_regs<kMain, true>(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
       }
       uint32_t total = 0;
       for (int lane = 0; lane < kLanes; ++lane) {
-        count[lane] = all_fit ? regs[lane].count
-                              : count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane]);
-        if (all_fit && force_check)   // the two routes must agree on the count
-          if (count[lane] != count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane])) return 7;
+        count[lane] = regs[lane].count;
+        if (regs[lane].overflow)
+          count[lane] += count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, regs[lane].resume);
+        // the register route and the counting pass over the whole chunk must agree
+        if (count[lane] != count_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane])) return 7;
         excl[lane] = total;
         total += count[lane];
       }
       const SubPlan p = plan_sub((int64_t)subpos[sub], total, n_elements, stage_cap);
-      bool replay = all_fit && !force_two_pass;
+      bool replay = !force_two_pass;
       for (int lane = 0; lane < kLanes; ++lane)
         replay = replay && thread_quota(excl[lane], count[lane], p.n_out) == count[lane];
       // Replay ORs into the staging area: it must be all zero here, which is the
@@ -183,10 +182,15 @@ static int emul_run(const uint8_t* luts, const uint8_t* codes, const uint8_t* si
       for (int k = 0; k < kLanes; ++k) {
         const int lane = (sub & 1) ? kLanes - 1 - k : k;
         const uint32_t quota = thread_quota(excl[lane], count[lane], p.n_out);
-        // a lane with nothing to write may hold an out-of-range pointer; it must not use it
-        uint8_t* dst = quota ? stage.p + p.phase + excl[lane] : nullptr;
-        if (replay) replay_chunk(regs[lane], stage_mem.p, (uint32_t)kLeadIn + p.phase + excl[lane]);
-        else emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota, dst);
+        const uint32_t at = (uint32_t)kLeadIn + p.phase + excl[lane];
+        if (replay) {
+          replay_chunk(regs[lane], stage_mem.p, at);
+          if (regs[lane].overflow)
+            emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, regs[lane].resume,
+                       count[lane] - regs[lane].count, stage_mem.p, at + regs[lane].count);
+        } else {
+          emit_chunk(t, l, chunk[lane].hi, chunk[lane].lo, chunk[lane].next, gap[lane], quota, stage_mem.p, at);
+        }
       }
       const SubSpans sp = spans_of(p);
       if (vec_ok) {
@@ -240,13 +244,22 @@ static int emul_run(const uint8_t* luts, const uint8_t* codes, const uint8_t* si
   return 0;
 }
 
+// flags: bit 0 forces the two-pass route on every sub-block; bits 8-9 select the
+// compilation by its register slots (0: the usual one, 1: the fewest, 2: short codes).
+#define DF11_EMUL_DISPATCH(...)                                                   \
+  switch ((flags >> 8) & 3) {                                                     \
+    case 1: return emul_run<kMainSlotsFew>(__VA_ARGS__);                          \
+    case 2: return emul_run<kMainSlotsShortCodes>(__VA_ARGS__);                   \
+    default: return emul_run<kMainSlotsUsual>(__VA_ARGS__);                       \
+  }
+
 extern "C" int df11_emul_decode(const uint8_t* luts, const uint8_t* codes, const uint8_t* sign_mantissa,
                                 const uint32_t* positions, const uint8_t* gaps, uint16_t* out,
                                 int n_luts, int64_t n_bytes, int64_t n_elements,
                                 int max_elems_per_sub, int grid, int codes_misalign,
                                 int out_misalign, int flags) {
-  return emul_run(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes, n_elements, max_elems_per_sub,
-                  grid, codes_misalign, out_misalign, flags, nullptr, 0, 0);
+  DF11_EMUL_DISPATCH(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes, n_elements, max_elems_per_sub,
+                     grid, codes_misalign, out_misalign, flags, nullptr, 0, 0)
 }
 
 // Host counterpart of df11_decode_rows; `out` holds the caller's buffer on entry.
@@ -255,8 +268,9 @@ extern "C" int df11_emul_decode_rows(const uint8_t* luts, const uint8_t* codes, 
                                      int n_luts, int64_t n_bytes, int64_t n_elements, int max_elems_per_sub,
                                      const int64_t* row_ids, int64_t n_ids, int64_t row_elements) {
   if (!row_ids || row_elements <= 0) return 1;
-  return emul_run(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes, n_elements, max_elems_per_sub,
-                  1, 0, 0, 0, row_ids, n_ids, row_elements);
+  const int flags = 0;
+  DF11_EMUL_DISPATCH(luts, codes, sign_mantissa, positions, gaps, out, n_luts, n_bytes, n_elements, max_elems_per_sub,
+                     1, 0, 0, flags, row_ids, n_ids, row_elements)
 }
 
 #ifdef DF11_EMUL_MAIN

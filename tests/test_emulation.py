@@ -31,20 +31,24 @@ def _p(a):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0, two_pass=False):
+SLOTS = {"usual": 0, "few": 1, "short": 2}
+
+
+def run_emul(L, c, max_elems=0, grid=3, codes_misalign=0, out_misalign=0, two_pass=False, slots="usual"):
+    """slots: which compilation's register slots to emulate (10, 7 or 14 lookups inside a chunk)."""
     n = c["sign_mantissa"].size
     out = np.zeros(n, np.uint16)
     luts = np.ascontiguousarray(c["luts"])
     rc = L.df11_emul_decode(_p(luts), _p(c["encoded_exponent"]), _p(c["sign_mantissa"]),
                             _p(c["output_positions"]), _p(c["gaps"]), _p(out), luts.shape[0],
                             c["encoded_exponent"].size, n, max_elems, grid, codes_misalign, out_misalign,
-                            1 if two_pass else 0)
+                            (1 if two_pass else 0) | (SLOTS[slots] << 8))
     assert rc == 0
     return out
 
 
 def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=None, two_pass=False,
-             ok_codes=(0,), rows=False):
+             ok_codes=(0,), rows=False, slots="usual"):
     """rows: df11_decode_rows for rows 6, 0, 3 of the output as a seven-row matrix (and numbers
     outside it) into a buffer of 0xEEEE, instead of the whole stream."""
     n = c["sign_mantissa"].size
@@ -54,7 +58,8 @@ def run_asan(c, max_elems=0, grid=2, codes_misalign=0, out_misalign=0, tmp_path=
     inp, outp = str(tmp_path / "case.bin"), str(tmp_path / "out.bin")
     with open(inp, "wb") as f:
         f.write(np.array([luts.shape[0], n_bytes, n, n_blocks, max_elems, grid, codes_misalign,
-                          out_misalign, (1 if two_pass else 0) | (4 if rows else 0)], np.int64).tobytes())
+                          out_misalign, (1 if two_pass else 0) | (4 if rows else 0) | (SLOTS[slots] << 8)],
+                         np.int64).tobytes())
         f.write(luts.tobytes())
         f.write(c["encoded_exponent"].tobytes())
         f.write(c["sign_mantissa"].tobytes())
@@ -78,6 +83,9 @@ def test_emulated_kernel_matches_oracle(emul, oracle, kind, n):
     assert np.array_equal(got, ref)
     # worst-case staging selected by max_elems <= 0; the two-pass fall-back route on every input
     assert np.array_equal(run_emul(emul, c, max_elems=0, grid=1, two_pass=True), ref)
+    # the compilations with other numbers of register slots
+    for slots in ("few", "short"):
+        assert np.array_equal(run_emul(emul, c, max_elems=0, grid=2, slots=slots), ref), slots
 
 
 @pytest.mark.parametrize("kind", ["normal", "zeros", "fib", "uniform256"])
@@ -157,6 +165,10 @@ def test_emulated_kernel_under_asan(emul, tmp_path, kind, n, cm, om):
         got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
                        out_misalign=om, tmp_path=tmp_path, two_pass=two_pass)
         assert np.array_equal(got, w)
+    for slots in ("few", "short"):
+        got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), codes_misalign=cm,
+                       out_misalign=om, tmp_path=tmp_path, slots=slots)
+        assert np.array_equal(got, w), slots
     got = run_asan(c, max_elems=max_elems_per_block(c["output_positions"]), tmp_path=tmp_path, rows=True)
     row = max(1, n // 7)
     for i in (6, 0, 3):
@@ -371,6 +383,8 @@ def test_emulated_kernel_random_codes_and_fillings(emul, oracle, chunk):
             assert np.array_equal(ref, w), (seed, policy)
             for two_pass in (False, True):
                 assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (seed, policy, two_pass)
+            for slots in ("few", "short"):
+                assert np.array_equal(run_emul(emul, c, slots=slots), w), (seed, policy, slots)
             ran += 1
     assert ran > 20
 
@@ -389,6 +403,31 @@ def test_emulated_kernel_every_lut_row(emul, oracle, n):
         assert np.array_equal(ref, w), policy
         for two_pass in (False, True):
             assert np.array_equal(run_emul(emul, c, two_pass=two_pass), w), (policy, two_pass)
+        for slots in ("few", "short"):
+            assert np.array_equal(run_emul(emul, c, slots=slots), w), (policy, slots)
+
+
+@pytest.mark.parametrize("slots", ["usual", "few", "short"])
+def test_emulated_kernel_chunks_of_many_lookups(emul, slots):
+    """Streams whose chunks need more lookups than weight-like ones: sparse weights (one- to
+    three-bit codes next to long ones, up to sixteen lookups of four codes) and alphabets of
+    48 to 240 equally likely exponents (six- to eight-bit codes, one per lookup, up to eleven).
+    Whatever the compilation's register slots hold or not, the output is the original words
+    (the emulation also compares the register route's counts with the counting pass)."""
+    rng = np.random.default_rng(11)
+    n = 120_000
+    sm = rng.integers(0, 256, n).astype(np.uint16)
+
+    def words(e):
+        return (((sm & 0x80) << 8) | (e.astype(np.uint16) << 7) | (sm & 0x7F)).astype(np.uint16)
+
+    for p_zero in (1.0, 0.97, 0.9, 0.7, 0.5):
+        e = np.where(rng.random(n) < p_zero, 0, np.clip(rng.normal(121, 2.5, n), 90, 135).astype(np.int64))
+        w = words(e)
+        assert np.array_equal(run_emul(emul, compress_product(w), grid=2, slots=slots), w), p_zero
+    for alphabet in (48, 64, 100, 128, 200, 240):
+        w = words(rng.integers(0, alphabet, n))
+        assert np.array_equal(run_emul(emul, compress_product(w), grid=2, slots=slots), w), alphabet
 
 
 def test_emulated_kernel_few_elements_many_symbols(emul, oracle):

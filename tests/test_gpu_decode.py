@@ -337,10 +337,11 @@ def test_gpu_llama_block_round_trip():
 
 
 @pytest.mark.parametrize("rows,cols", [(151936, 4096), (4096, 14336)])
-@pytest.mark.parametrize("kind", ["laplace", "outliers", "uniform256", "zeros"])
+@pytest.mark.parametrize("kind", ["laplace", "outliers", "uniform256", "zeros", "sparse70", "alphabet100"])
 def test_gpu_embedding_sized_adversarial_round_trip(kind, rows, cols):
     """151936 x 4096 (622 329 856 elements, the largest tensor of the Qwen3-8B shape) and
-    4096 x 14336 with an adversarial exponent mix: encode -> decode is the identity."""
+    4096 x 14336 with an adversarial exponent mix (the last two: chunks of thirty and more
+    codes, and of nine to eleven table lookups): encode -> decode is the identity."""
     print(f"case {rows}x{cols} {kind}", flush=True)
     import bench_extra
     w = bench_extra.make_mix(torch, kind, rows * cols, torch.device(DEV), seed=23)
