@@ -155,8 +155,9 @@ int df11_decode_static_workspace(const uint8_t *luts, const uint8_t *encoded_exp
  * compiled for three launch plans (workgroups resident per CU and how far ahead
  * it requests sign_mantissa bytes: DF11_PLAN_WIDE, _DEEP, _DEEPEST; the two plans
  * for large streams come in further compilations that differ in how wavefront
- * priorities are set and in the cache policy of the loads, which the stream's
- * size decides in either entry point), seven kernels in all with
+ * priorities are set and in the cache policy of the loads, and `wide` in two more
+ * with four workgroups per CU, which the stream's size and code lengths decide
+ * when the plan is left to the library), nine kernels in all with
  * DF11_PLAN_PORTABLE.  df11_decode picks the plan per stream from its size and
  * its elements per 512 bytes of bitstream; this entry point takes it as an
  * argument, for tests that drive every stream through every plan and for
@@ -183,7 +184,8 @@ int df11_decode_with_plan(const uint8_t *luts, const uint8_t *encoded_exponent,
  * Which compilation of the decode kernel df11_decode launches for a stream of
  * n_bytes of encoded_exponent and n_elements on a device of compute_units CUs
  * (when the LDS the stream needs leaves room for the plan's workgroups per CU):
- * "wide", "deep", "deep/short", "deep/small", "deepest" or "deepest/short";
+ * "wide", "wide/full", "wide/dense", "deep", "deep/short", "deep/small", "deepest"
+ * or "deepest/short";
  * "" for sizes that are not positive.  Needs no GPU.  Testing aid with no
  * counterpart in the reference.
  */
