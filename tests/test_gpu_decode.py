@@ -277,6 +277,45 @@ def test_gpu_side_stream_and_repeat():
     assert np.array_equal(b.view(torch.int16).cpu().numpy().view(np.uint16), w2)
 
 
+def test_gpu_host_threads_decode_at_once():
+    """The library keeps no launch state between calls: host threads that prepare and decode
+    streams of their own at the same time, each on a stream of its own, all get their words."""
+    import threading
+    print("case host threads", flush=True)
+    specs = [("normal", 400_003, 5), ("zeros", 250_000, 6), ("uniform256", 120_001, 7), ("sparse", 300_000, 8)]
+    cases = [(make_case(kind, n, seed), kind) for kind, n, seed in specs]
+    packed = [(w, to_gpu(compress_product(w))) for w, _ in cases]
+    torch.cuda.synchronize()
+    results, errors = [None] * len(packed), []
+
+    def work(i):
+        try:
+            torch.cuda.set_device(0)
+            w, g = packed[i]
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                good = True
+                for _ in range(8):
+                    ws, max_sub = D.prepare(g["luts"].contiguous(), g["encoded_exponent"], g["output_positions"],
+                                            g["gaps"], w.size)
+                    out = torch.full((w.size,), float("nan"), dtype=torch.bfloat16, device=DEV)
+                    D.decode(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"],
+                             g["gaps"], out, ws, max_sub)
+                    s.synchronize()
+                    good = good and np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), w)
+            results[i] = good
+        except Exception as e:   # reported by the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(packed))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(100)
+    assert not errors, errors
+    assert results == [True] * len(packed), results
+
+
 def test_gpu_decode_in_a_captured_graph():
     """df11_decode allocates nothing and never synchronises, so it can be captured into
     a HIP graph; every replay (with eager work and synchronisation between replays)
