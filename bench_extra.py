@@ -14,6 +14,10 @@
                            compressed streams live in pinned host memory and are copied
                            one block ahead of use; per-block copy+decode latency, peak
                            device memory, outputs against the non-offloaded run
+  --workload rows          df11_decode_rows on the 151936x4096 embedding table of the
+                           Qwen3-8B shape: time per launch for 1 to 32768 looked-up rows
+                           against the decode of the whole table, rows checked against
+                           the original words
 """
 import argparse
 import json
@@ -168,6 +172,57 @@ def run_mixes(a, torch, dev):
             torch.cuda.empty_cache()
             ok = ok and r["bit_exact"]
             print(json.dumps({"workload": "mixes", "mix": kind, "tensor": f"{name} {rows}x{cols}", **r}), flush=True)
+    return ok
+
+
+ROW_COUNTS = (1, 8, 64, 512, 4096, 32768)
+
+
+def run_rows(a, torch, dev):
+    """The embedding lookup's decode: only the rows that the ids name (the reference decodes
+    the whole table before every lookup: dfloat11.py:153-157)."""
+    from dfloat11_amd import decode as D
+    from dfloat11_amd import dfloat11_utils as U
+    rows, cols = MIX_SHAPES[0][1:]
+    w = make_mix(torch, "normal", rows * cols, dev, seed=7)
+    w_cpu = w.cpu()
+    _, counter = U.get_codec(w_cpu)
+    codec, _, table = U.get_32bit_codec(counter)
+    luts = U.get_luts(table)
+    enc, sm, pos, gaps, _ = U.encode_weights([w_cpu], codec)
+    del w_cpu
+    d = [t.to(dev) for t in (luts, enc, sm)] + [pos.view(torch.uint8).to(dev), gaps.to(dev)]
+    ws, max_sub = D.prepare(d[0], d[1], d[3], d[4], rows * cols)
+    out = torch.empty(rows * cols, dtype=torch.bfloat16, device=dev)
+    bound = D.bind(d[0], d[1], d[2], d[3], d[4], out, ws, max_sub)
+
+    def per_launch_us(launch, n=50):
+        for _ in range(10):
+            launch()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(n):
+            launch()
+        t1.record()
+        torch.cuda.synchronize()
+        return t0.elapsed_time(t1) / n * 1e3
+
+    whole_us = per_launch_us(lambda: D.launch(bound, dev))
+    ok = bool(torch.equal(out.view(torch.int16), w.view(torch.int16)))
+    print(json.dumps({"workload": "rows", "tensor": f"embedding {rows}x{cols}", "rows_decoded": "all",
+                      "us_per_launch": whole_us, "bit_exact": ok}), flush=True)
+    g = torch.Generator().manual_seed(0)
+    for n_ids in ROW_COUNTS:
+        ids = torch.randint(0, rows, (n_ids,), generator=g).to(dev)
+        out.zero_()
+        D.launch_rows(bound, dev, ids, cols)
+        torch.cuda.synchronize()
+        exact = bool(torch.equal(out.view(rows, cols)[ids].view(torch.int16), w.view(rows, cols)[ids].view(torch.int16)))
+        ok = ok and exact
+        print(json.dumps({"workload": "rows", "tensor": f"embedding {rows}x{cols}", "rows_decoded": n_ids,
+                          "us_per_launch": per_launch_us(lambda: D.launch_rows(bound, dev, ids, cols)),
+                          "bit_exact": exact}), flush=True)
     return ok
 
 
@@ -383,7 +438,7 @@ def run_flux(a, torch, dev):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--workload", choices=["mixes", "sizes", "flux-offload"], required=True)
+    ap.add_argument("--workload", choices=["mixes", "sizes", "flux-offload", "rows"], required=True)
     ap.add_argument("--mix", choices=MIXES + EXTRA_MIXES + ("normal",), default=None, help="mixes: only this distribution")
     ap.add_argument("--tensor", choices=[t[0] for t in ALL_SHAPES], default=None, help="mixes: only this tensor")
     ap.add_argument("--regime", choices=["hbm", "cache", "both"], default="both",
@@ -399,7 +454,7 @@ def main():
         sys.exit("bench_extra.py needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    ok = {"mixes": run_mixes, "sizes": run_sizes, "flux-offload": run_flux}[a.workload](a, torch, dev)
+    ok = {"mixes": run_mixes, "sizes": run_sizes, "flux-offload": run_flux, "rows": run_rows}[a.workload](a, torch, dev)
     sys.exit(0 if ok else 1)
 
 
