@@ -9,7 +9,14 @@ import torch
 from . import _native
 
 
+# The handle of a device's current stream without building a torch.cuda.Stream object
+# around it (the hook asks for it before every launch).
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(device):
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -166,9 +173,12 @@ def launch_rows(bound, device, row_ids, row_elements):
     if row_ids.dtype != torch.int64 or row_ids.device != device or not row_ids.is_contiguous():
         raise _native.DF11Error("row_ids must be a contiguous int64 tensor on the stream's device")
     lib = _native.hip_lib()
-    with torch.cuda.device(device):
-        rc = lib.df11_decode_rows(*bound, torch.cuda.current_stream(device).cuda_stream,
-                                  row_ids.data_ptr(), row_ids.numel(), int(row_elements))
+    if torch.cuda.current_device() == device.index:
+        rc = lib.df11_decode_rows(*bound, _stream_ptr(device), row_ids.data_ptr(), row_ids.numel(), int(row_elements))
+    else:
+        with torch.cuda.device(device):
+            rc = lib.df11_decode_rows(*bound, _stream_ptr(device), row_ids.data_ptr(), row_ids.numel(),
+                                      int(row_elements))
     if rc:
         _native.check(rc, "df11_decode_rows")
 
@@ -177,9 +187,9 @@ def launch(bound, device):
     """df11_decode with arguments from bind(), on the current stream of `device`."""
     lib = _native.hip_lib()
     if torch.cuda.current_device() == device.index:
-        rc = lib.df11_decode(*bound, torch.cuda.current_stream(device).cuda_stream)
+        rc = lib.df11_decode(*bound, _stream_ptr(device))
     else:
         with torch.cuda.device(device):
-            rc = lib.df11_decode(*bound, torch.cuda.current_stream(device).cuda_stream)
+            rc = lib.df11_decode(*bound, _stream_ptr(device))
     if rc:
         _native.check(rc, "df11_decode")
