@@ -536,23 +536,37 @@ __device__ __forceinline__ void decode_body(
   };
 
   if (kRows) {
-    // Workgroup i takes ids i, i + grid, ...; its eight wavefronts take the sub-blocks
-    // that overlap the id's elements in turn.  Each sub-block is written out whole, so
-    // the elements next to a row, up to a sub-block's worth on either side, are decoded
-    // with it (to the same values any other decode of them writes).
+    // Up to as many ids as there are workgroups, workgroup i takes id i and its eight
+    // wavefronts take the sub-blocks that overlap the id's elements in turn: one round, the
+    // shortest way to the few rows of a generation step.  With more ids every wavefront
+    // takes ids of its own and walks a row's sub-blocks by itself, eight times as many rows
+    // in flight.  Either way the next sub-block's inputs are requested a step ahead, and each
+    // sub-block is written out whole, so the elements next to a row, up to a sub-block's
+    // worth on either side, are decoded with it (to the same values any other decode of
+    // them writes).
     const uint32_t n_entries = (uint32_t)(z.n_blocks * kSubsPerBlock + 1);
     const int64_t n_rows_total = rows.row_elements > 0 ? z.n_elements / rows.row_elements : 0;
-    for (int64_t i = blockIdx.x; i < rows.n_ids; i += gridDim.x) {
+    const bool id_per_wave = rows.n_ids > (int64_t)gridDim.x;      // uniform
+    const int64_t first_id = id_per_wave ? (int64_t)blockIdx.x * kWavesPerGroup + wave : (int64_t)blockIdx.x;
+    const int64_t id_stride = id_per_wave ? (int64_t)gridDim.x * kWavesPerGroup : (int64_t)gridDim.x;
+    const int64_t first_sub = id_per_wave ? 0 : (int64_t)wave;
+    const int64_t sub_stride = id_per_wave ? 1 : kWavesPerGroup;
+    for (int64_t i = first_id; i < rows.n_ids; i += id_stride) {
       const int64_t id = rows.ids[i];                         // uniform
       if (id < 0 || id >= n_rows_total) continue;             // ids outside the matrix select nothing
       const int64_t first = id * rows.row_elements;
       const int64_t end = first + rows.row_elements;
-      const uint32_t s0 = uniform(find_sub(subpos, n_entries, (uint32_t)first, lane));
-      for (int64_t s = (int64_t)s0 + wave; s < z.n_subs; s += kWavesPerGroup) {
-        SubInputs in = fetch_sub<kStreaming>(codes, gaps, subpos, z, s, lane, gap_byte, vzero);
+      int64_t s = (int64_t)uniform(find_sub(subpos, n_entries, (uint32_t)first, lane)) + first_sub;
+      if (s >= z.n_subs) continue;
+      SubInputs in = fetch_sub<kStreaming>(codes, gaps, subpos, z, s, lane, gap_byte, vzero);
+      for (;;) {
         if ((int64_t)uniform(in.base) >= end) break;          // starts past the row
         claim(in.d0, in.d1, in.d2, in.gap_raw, in.base, in.end_hint);
-        step(in, false, 0);
+        const int64_t next = s + sub_stride;
+        const bool more = next < z.n_subs;
+        in = step(in, more, next);
+        if (!more) break;
+        s = next;
       }
     }
     return;
@@ -614,7 +628,8 @@ DF11_DECODE_KERNEL(decode_kernel_wide_dense, 2, false, false, 8, true, kMainSlot
 
 // Decodes only the sub-blocks that hold given rows of the output matrix (an embedding
 // looks up a few rows of a table whose stream holds them all): `wide` settings, wavefront
-// priorities by phase, work taken per id instead of per sub-block.
+// priorities by phase, work taken per id (by a workgroup, or by a wavefront when the ids
+// outnumber the workgroups) instead of per sub-block.
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(6, 6)))
 void decode_kernel_rows(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ sign_mantissa,
                         const uint8_t* __restrict__ gaps, uint16_t* __restrict__ out,

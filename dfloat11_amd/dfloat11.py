@@ -285,7 +285,7 @@ def _looked_up_rows(module, inputs, device):
         return None
     ids = inputs[0]
     if ids.dtype != torch.int64 or ids.device != device or ids.numel() == 0 \
-            or ids.numel() * 8 > module.num_embeddings:
+            or ids.numel() * 4 > module.num_embeddings:
         return None
     return ids if ids.is_contiguous() else ids.contiguous()
 
