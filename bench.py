@@ -211,7 +211,7 @@ def main():
     ap.add_argument("--no-mixes", action="store_true",
                     help="skip the per-distribution and per-size side measurements (config.mixes, config.sizes)")
     ap.add_argument("--no-embedding-mixes", action="store_true",
-                    help="config.mixes on the 4096x14336 matrix only, not on the 151936x4096 tensor as well")
+                    help="config.mixes on the 4096x14336 matrix only, not on the 151936x4096 tensor as well, and no config.rows")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip config.e2e: Qwen3-8B-shaped generation, BF16 against DF11, batch 1 and 64 (about 1 min)")
     ap.add_argument("--e2e-tokens", type=int, default=64, help="new tokens per sequence in config.e2e")
@@ -412,6 +412,14 @@ def main():
                    + list(result["config"]["sizes"].values())):
             result["error"] = "a side measurement did not decode bit-exactly"
             bit_exact = False
+        if not a.no_embedding_mixes:
+            # the embedding's lookup: only the rows of the ids (df11_decode_rows) against the whole table
+            import bench_extra
+            result["config"]["rows"] = rows = bench_extra.measure_rows(torch, dev, row_counts=(1, 64, 4096))
+            torch.cuda.empty_cache()
+            if not all(r["bit_exact"] for r in rows):
+                result["error"] = "a row decode differs from the original rows"
+                bit_exact = False
     if not a.no_cpu_baseline:
         stream = dict(luts=luts.numpy(), encoded_exponent=enc.numpy(), sign_mantissa=sm.numpy(),
                       output_positions=pos.numpy(), gaps=gaps.numpy())

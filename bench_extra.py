@@ -178,9 +178,10 @@ def run_mixes(a, torch, dev):
 ROW_COUNTS = (1, 8, 64, 512, 4096, 32768)
 
 
-def run_rows(a, torch, dev):
+def measure_rows(torch, dev, row_counts=ROW_COUNTS):
     """The embedding lookup's decode: only the rows that the ids name (the reference decodes
-    the whole table before every lookup: dfloat11.py:153-157)."""
+    the whole table before every lookup: dfloat11.py:153-157).  One record for the whole
+    table through df11_decode, then one per id count through df11_decode_rows."""
     from dfloat11_amd import decode as D
     from dfloat11_amd import dfloat11_utils as U
     rows, cols = MIX_SHAPES[0][1:]
@@ -209,20 +210,26 @@ def run_rows(a, torch, dev):
         return t0.elapsed_time(t1) / n * 1e3
 
     whole_us = per_launch_us(lambda: D.launch(bound, dev))
-    ok = bool(torch.equal(out.view(torch.int16), w.view(torch.int16)))
-    print(json.dumps({"workload": "rows", "tensor": f"embedding {rows}x{cols}", "rows_decoded": "all",
-                      "us_per_launch": whole_us, "bit_exact": ok}), flush=True)
+    records = [{"tensor": f"embedding {rows}x{cols}", "rows_decoded": "all", "us_per_launch": whole_us,
+                "bit_exact": bool(torch.equal(out.view(torch.int16), w.view(torch.int16)))}]
     g = torch.Generator().manual_seed(0)
-    for n_ids in ROW_COUNTS:
+    for n_ids in row_counts:
         ids = torch.randint(0, rows, (n_ids,), generator=g).to(dev)
         out.zero_()
         D.launch_rows(bound, dev, ids, cols)
         torch.cuda.synchronize()
         exact = bool(torch.equal(out.view(rows, cols)[ids].view(torch.int16), w.view(rows, cols)[ids].view(torch.int16)))
-        ok = ok and exact
-        print(json.dumps({"workload": "rows", "tensor": f"embedding {rows}x{cols}", "rows_decoded": n_ids,
-                          "us_per_launch": per_launch_us(lambda: D.launch_rows(bound, dev, ids, cols)),
-                          "bit_exact": exact}), flush=True)
+        records.append({"tensor": f"embedding {rows}x{cols}", "rows_decoded": n_ids,
+                        "us_per_launch": per_launch_us(lambda: D.launch_rows(bound, dev, ids, cols)),
+                        "bit_exact": exact})
+    return records
+
+
+def run_rows(a, torch, dev):
+    ok = True
+    for r in measure_rows(torch, dev):
+        ok = ok and r["bit_exact"]
+        print(json.dumps({"workload": "rows", **r}), flush=True)
     return ok
 
 
