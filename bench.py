@@ -142,7 +142,7 @@ def end_to_end(torch, dev, num_tokens, batch_sizes=(1, 64)):
     t0 = time.perf_counter()
     out = {}
     for r in inference.compare_synthetic("qwen3-8b", list(batch_sizes), num_tokens, prompt_len=64, device=dev,
-                                         repeats=3):
+                                         repeats=5):
         out[f"batch {r['batch_size']}"] = {
             "new_tokens": r["num_tokens"], "prompt_len": r["prompt_len"], "timed_runs": r["df11"]["timed_runs"],
             "bf16_tokens_per_second": r["bf16"]["tokens_per_second"],
