@@ -138,57 +138,62 @@ def _random_prompts(model, batch_size, prompt_len, seed, device):
     return {"input_ids": ids, "attention_mask": torch.ones_like(ids)}
 
 
-def _median_run(model, inputs, num_tokens, repeats):
-    """timed_generate `repeats` times; the run of median latency and its output."""
-    runs = [timed_generate(model, inputs, num_tokens, False) for _ in range(max(1, repeats))]
-    runs.sort(key=lambda r: r[1]["latency_s"])
-    out, stats = runs[len(runs) // 2]
-    stats["timed_runs"] = len(runs)
-    return out, stats
-
-
 def compare_synthetic(shape, batch_sizes, num_tokens, prompt_len=64, seed=42, device="cuda:0", layers=None,
                       repeats=1):
-    """Builds the named architecture once with random-init BF16 weights, generates
-    greedily at every batch size, compresses the model in memory and generates again
-    from the same prompts.  Returns one report per batch size with the fields of the
-    reference's benchmark for both models (reference: inference.py:62-97), their
-    ratio, and whether logits and tokens are identical.  With repeats > 1 every figure is
-    the run of median latency out of that many (generation speed of the eager model varies
-    by several per cent from run to run on the same box)."""
+    """Builds the named architecture once with random-init BF16 weights, compresses a copy
+    of it in memory, and generates greedily from the same prompts with both at every batch
+    size.  Returns one report per batch size with the fields of the reference's benchmark
+    for both models (reference: inference.py:62-97), their ratio, and whether logits and
+    tokens are identical.  The timed runs of the two models alternate (BF16, DF11, BF16, ...,
+    `repeats` of each) and each model reports its run of median latency: generation speed of
+    the eager model drifts by several per cent over a minute on the same box, and runs taken
+    one model after the other would put that drift into the ratio.  Both models are resident
+    throughout, so each model's memory figures are what the device holds minus the other
+    model's share."""
+    import copy
     import torch
     device = torch.device(device)
     model = build_synthetic(shape, device, seed, layers)
     name = f"{shape} (random-init N(0, 0.02), {sum(p.numel() for p in model.parameters())/1e9:.2f} B parameters)"
-    reports, kept = [], []
+    bf16_bytes = torch.cuda.memory_allocated(device)
+    df11_model = copy.deepcopy(model)
+    t0 = time.time()
+    compressed, original = convert_in_memory(df11_model, LLM_PATTERNS, device)
+    compress_seconds = time.time() - t0
+    torch.cuda.empty_cache()
+    reports = []
     for b in batch_sizes:
         inputs = _random_prompts(model, b, prompt_len, seed, device)
         with torch.no_grad():
             ref_logits = model(**inputs, use_cache=False).logits
-        timed_generate(model, inputs, min(8, num_tokens), False)           # warm-up
-        ref_out, stats = _median_run(model, inputs, num_tokens, repeats)
-        reports.append({"batch_size": b, "num_tokens": num_tokens, "model": name, "prompt_len": prompt_len,
-                        "bf16": stats})
-        kept.append((inputs, ref_logits.cpu(), ref_out))
-        del ref_logits
-    t0 = time.time()
-    compressed, original = convert_in_memory(model, LLM_PATTERNS, device)
-    compress_seconds = time.time() - t0
-    torch.cuda.empty_cache()
-    for report, (inputs, ref_logits, ref_out) in zip(reports, kept):
-        report["compress_seconds"] = compress_seconds
-        report["compressed_over_bf16"] = compressed / original
-        # warm-up pass: first-use work (decode workspaces, library handles) stays out of the timing
-        with torch.no_grad():
-            logits = model(**inputs, use_cache=False).logits
+            # also the DF11 model's warm-up pass: first-use work (decode workspaces, library
+            # handles) stays out of the timing
+            logits = df11_model(**inputs, use_cache=False).logits
+        logits_identical = bool(torch.equal(logits, ref_logits))
+        del logits, ref_logits
         timed_generate(model, inputs, min(8, num_tokens), False)
-        out, stats = _median_run(model, inputs, num_tokens, repeats)
-        report["df11"] = stats
-        report["logits_bit_identical"] = bool(torch.equal(logits.cpu(), ref_logits))
-        report["tokens_identical"] = bool(torch.equal(out, ref_out))
-        report["df11_over_bf16_tokens_per_second"] = stats["tokens_per_second"] / report["bf16"]["tokens_per_second"]
-        del logits
-    del model
+        timed_generate(df11_model, inputs, min(8, num_tokens), False)
+        df11_bytes = torch.cuda.memory_allocated(device) - bf16_bytes      # streams, shared buffer, workspaces
+        runs = {"bf16": [], "df11": []}
+        for _ in range(max(1, repeats)):
+            runs["bf16"].append(timed_generate(model, inputs, num_tokens, False))
+            runs["df11"].append(timed_generate(df11_model, inputs, num_tokens, False))
+        report = {"batch_size": b, "num_tokens": num_tokens, "model": name, "prompt_len": prompt_len,
+                  "compress_seconds": compress_seconds, "compressed_over_bf16": compressed / original,
+                  "logits_bit_identical": logits_identical}
+        outs = {}
+        for which, other_bytes in (("bf16", df11_bytes), ("df11", bf16_bytes)):
+            ordered = sorted(runs[which], key=lambda r: r[1]["latency_s"])
+            outs[which], stats = ordered[len(ordered) // 2]
+            stats = dict(stats, timed_runs=len(ordered))
+            for key in ("gpu_memory_allocated_mb", "gpu_peak_memory_mb"):
+                stats[key] -= other_bytes / 1e6
+            report[which] = stats
+        report["tokens_identical"] = bool(torch.equal(outs["df11"], outs["bf16"]))
+        report["df11_over_bf16_tokens_per_second"] = (report["df11"]["tokens_per_second"]
+                                                      / report["bf16"]["tokens_per_second"])
+        reports.append(report)
+    del model, df11_model
     from . import dfloat11 as D
     D.TensorManager.clear()
     torch.cuda.empty_cache()
