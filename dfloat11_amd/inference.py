@@ -230,6 +230,8 @@ def main(argv=None):
     ap.add_argument("--greedy", action="store_true", help="greedy decoding (default for --synthetic)")
     ap.add_argument("--compare_bf16", action="store_true",
                     help="--synthetic only: run the BF16 model first, then its DF11 form, and compare")
+    ap.add_argument("--repeats", type=int, default=1,
+                    help="--compare_bf16 only: timed generations per model, alternating; the median run is reported")
     ap.add_argument("--device", type=str, default="cuda:0")
     ap.add_argument("--json", action="store_true", help="print one JSON line instead of the text report")
     a = ap.parse_args(argv)
@@ -244,7 +246,7 @@ def main(argv=None):
 
     if a.synthetic and a.compare_bf16:
         report = compare_synthetic(a.synthetic, [a.batch_size], a.num_tokens, a.prompt_len, a.seed, device,
-                                   a.layers)[0]
+                                   a.layers, a.repeats)[0]
         _print_report(report, a.json)
         return report
     if a.synthetic:
