@@ -342,6 +342,48 @@ def test_gpu_decode_in_a_captured_graph():
         assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), w)
 
 
+def test_gpu_row_decode_in_a_captured_graph():
+    """df11_decode_rows reads the row numbers from device memory when it runs, so a graph
+    that captured one launch decodes whatever rows the caller has written into that buffer
+    by the time of each replay (also more rows than workgroups, where every wavefront takes
+    ids of its own)."""
+    print("case graph capture rows", flush=True)
+    n_rows, row_elements = 6000, 160
+    w = make_case("normal", n_rows * row_elements, 133)
+    c = compress_product(w)
+    g = to_gpu(c)
+    ws, max_sub = D.prepare(g["luts"], g["encoded_exponent"], g["output_positions"], g["gaps"], w.size)
+    sentinel = 0x7F81                        # a NaN pattern no stream of these kinds holds
+    out = torch.full((w.size,), sentinel, dtype=torch.int16, device=DEV).view(torch.bfloat16)
+    ids = torch.zeros(3000, dtype=torch.int64, device=DEV)
+    bound = D.bind(g["luts"], g["encoded_exponent"], g["sign_mantissa"], g["output_positions"], g["gaps"],
+                   out, ws, max_sub)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        D.launch_rows(bound, torch.device(DEV), ids, row_elements)   # warm-up outside the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        D.launch_rows(bound, torch.device(DEV), ids, row_elements)
+    rng = np.random.default_rng(5)
+    matrix = w.reshape(n_rows, row_elements)
+    for replay in range(4):
+        chosen = rng.integers(0, n_rows, ids.numel())
+        if replay == 3:
+            chosen[:] = chosen[0]            # one row, asked for 3000 times
+        out.view(torch.int16).fill_(sentinel)                        # eager work between the replays
+        ids.copy_(torch.from_numpy(chosen))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.view(torch.int16).cpu().numpy().view(np.uint16).reshape(n_rows, row_elements)
+        assert np.array_equal(got[chosen], matrix[chosen]), replay
+        written = got != sentinel
+        assert np.array_equal(got[written], matrix[written]), replay
+        if replay == 3:
+            assert written.sum() < 3 * 4096 + row_elements, replay    # the row and its sub-blocks' neighbours only
+
+
 def test_gpu_full_size_linear_round_trip():
     """4096x4096 N(0, 0.02): encode -> decode is the identity (size-independent property)."""
     print("case 4096x4096", flush=True)
@@ -445,7 +487,8 @@ def test_gpu_rows_match_full_decode(oracle, kind, n_rows, row_elements):
     """df11_decode_rows writes the requested rows exactly as df11_decode (and the oracle)
     does, writes nothing but correct values anywhere else, and leaves elements that are far
     from every requested row alone.  Row numbers repeat, come unsorted, include the first
-    and the last row and numbers outside the matrix."""
+    and the last row and numbers outside the matrix; they are fewer and more than the
+    workgroups of a launch (the kernel hands them out differently)."""
     n = n_rows * row_elements
     print(f"case rows kind={kind} rows={n_rows} row_elements={row_elements}", flush=True)
     w = make_case(kind, n, 91)
@@ -455,7 +498,7 @@ def test_gpu_rows_match_full_decode(oracle, kind, n_rows, row_elements):
     g = to_gpu(c)
     ws, max_sub = D.prepare(g["luts"].contiguous(), g["encoded_exponent"], g["output_positions"], g["gaps"], n)
     rng = np.random.default_rng(17)
-    for n_ids in (1, 5, 64):
+    for n_ids in (1, 5, 64, 2000):           # the last: more ids than workgroups, a wavefront per id
         ids = rng.integers(0, n_rows, n_ids)
         ids[0] = n_rows - 1
         if n_ids > 2:
