@@ -14,6 +14,10 @@ class DF11Error(RuntimeError):
     pass
 
 
+ERR_UNSUPPORTED = -2    # DF11_ERR_UNSUPPORTED
+ERR_HIP = -3            # DF11_ERR_HIP
+
+
 def codec_lib():
     """Host codec library (no GPU needed)."""
     global _codec
@@ -70,6 +74,6 @@ def check(rc, what):
         msg = f"{what} failed with code {rc}"
         if L is not None:
             msg += f" ({L.df11_error_string(rc).decode()})"
-            if rc == -3:
+            if rc == ERR_HIP:
                 msg += f": {L.df11_last_hip_error().decode()}"
         raise DF11Error(msg)

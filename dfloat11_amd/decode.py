@@ -162,14 +162,18 @@ def decode_rows(luts, encoded_exponent, sign_mantissa, output_positions, gaps, o
     matrix of row_elements elements per row, into their places in `out` (full size)."""
     bound = bind(luts, encoded_exponent, sign_mantissa, output_positions, gaps, out, workspace,
                  max_elems_per_subblock)
-    launch_rows(bound, out.device, row_ids, row_elements)
+    if not launch_rows(bound, out.device, row_ids, row_elements):
+        raise _native.DF11Error("df11_decode_rows is not available on this device; decode the whole stream")
     return out
 
 
 def launch_rows(bound, device, row_ids, row_elements):
     """df11_decode_rows with arguments from bind(): decodes the rows of the output matrix
     (row_elements elements each) that the int64 device tensor `row_ids` names, into
-    their places in the bound output buffer; the rest of the buffer is left as it is."""
+    their places in the bound output buffer; the rest of the buffer is left as it is.
+    Returns False, with nothing launched, if the library has no row decode for this
+    device (it then runs every stream through its portable kernel): the caller decodes
+    the whole stream instead."""
     if row_ids.dtype != torch.int64 or row_ids.device != device or not row_ids.is_contiguous():
         raise _native.DF11Error("row_ids must be a contiguous int64 tensor on the stream's device")
     lib = _native.hip_lib()
@@ -179,8 +183,11 @@ def launch_rows(bound, device, row_ids, row_elements):
         with torch.cuda.device(device):
             rc = lib.df11_decode_rows(*bound, _stream_ptr(device), row_ids.data_ptr(), row_ids.numel(),
                                       int(row_elements))
+    if rc == _native.ERR_UNSUPPORTED:
+        return False
     if rc:
         _native.check(rc, "df11_decode_rows")
+    return True
 
 
 def launch(bound, device):

@@ -315,9 +315,7 @@ def get_hook(threads_per_block, bytes_per_thread):
         if plan is not None and plan[0] is TensorManager._tensors.get(device) \
                 and _same_streams(module, plan[1]) and _views_in_place(plan[3]):
             row_ids = _looked_up_rows(module, inputs, device) if plan[4] else None
-            if row_ids is not None:
-                _decode.launch_rows(plan[2], device, row_ids, plan[4])
-            else:
+            if row_ids is None or not _decode.launch_rows(plan[2], device, row_ids, plan[4]):
                 _decode.launch(plan[2], device)
             return
 

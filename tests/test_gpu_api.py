@@ -410,3 +410,12 @@ def test_embedding_decodes_only_the_rows_it_looks_up(tmp_path):
             assert torch.equal(model.embed.weight, ref_weight)
         finally:
             M.EMBEDDING_ROW_DECODE = True
+        # a library that has no row decode for the device says so and the hook decodes the whole table
+        real = M._decode.launch_rows
+        M._decode.launch_rows = lambda *args: False
+        try:
+            buf.view(torch.int16).fill_(0x1234)
+            assert torch.equal(model(ids), ref_weight[ids])
+            assert torch.equal(model.embed.weight, ref_weight)
+        finally:
+            M._decode.launch_rows = real
